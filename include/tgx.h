@@ -27,7 +27,8 @@ extern "C" {
 
 /* 3 (round 5): per-row sequence lifecycle (tgx_reset_row / tgx_forward_row / tgx_sample_row / tgx_past_length_row); tgx_get_option added and
  * tgx_engine_read_stats + the options engine.*, pf.*, attn.fold_*, lmhead.fuse_finalize removed since 2. */
-#define TGX_ABI_VERSION 5   /* 4: layered models (tgx_create_stack, tgx_step_ragged); 5: Modepel (more mixers / feed-forward kinds in tgx_layer_desc) */
+#define TGX_ABI_VERSION 6   /* 4: layered models (tgx_create_stack, tgx_step_ragged); 5: Modepel (more mixers / feed-forward kinds in tgx_layer_desc);
+                             * 6: Vitudra (masks, score bias and cap, shared key / value layers, two recurrent mixers, parallel sublayers) */
 
 #if defined(__GNUC__)
 #define TGX_API __attribute__((visibility("default")))
@@ -57,7 +58,9 @@ typedef enum tgx_family {
   TGX_FAMILY_QWEN3 = 4,
   TGX_FAMILY_MISTRAL = 5,
   TGX_FAMILY_ZAKUSUN = 6,  /* a layered model (tgx_stack_desc below), no counterpart in the reference */
-  TGX_FAMILY_MODEPEL = 7   /* a layered model: rotary grouped-query attention and matrix-memory (mLSTM) layers, sandwich norms */
+  TGX_FAMILY_MODEPEL = 7,  /* a layered model: rotary grouped-query attention and matrix-memory (mLSTM) layers, sandwich norms */
+  TGX_FAMILY_VITUDRA = 8   /* a layered model: one norm per layer in front of a mixer and a gated feed-forward that run side by side; windowed and chunked
+                            * attention, shared key / value layers, decaying matrix states (token-shift "wkv" and gated delta rule) */
 } tgx_family;
 
 /* tinytorch::DType values the CLI accepts (examples/inference/main.cpp:82-88) */
@@ -117,8 +120,22 @@ typedef struct tgx_model_desc {
  *   dense feed-forward        down(PolyNorm(up(h))): a N(z) + b N(z^2) + c N(z^3) + e over a token's ff values
  *   grouped-choice experts    softmax router over experts + identity outputs; the choice adds a correction and is limited to the best groups_keep of
  *                             `groups` neighbour groups; weights = scores * router_scale; identity outputs hand the input through; gated-silu
- *                             experts; a shared expert of width shared_ff with a per-token sigmoid gate */
-typedef enum tgx_mixer { TGX_MIXER_LATENT_ATTENTION = 1, TGX_MIXER_ATTENTION = 2, TGX_MIXER_MLSTM = 3 } tgx_mixer;
+ *                             experts; a shared expert of width shared_ff with a per-token sigmoid gate
+ * and, for TGX_FAMILY_VITUDRA (x <- x + residual_mult * (mixer(h) + ff(h)), h = x / sqrt(mean(x^2) + norm_eps) * (1 + w); slots hold pages of the
+ * attention layers' key / value pools, one matrix state per recurrent head, the token-shift row and the convolution tails):
+ *   attention masks           mask_kind 1: a sliding window (position i sees j with 0 <= i - j < mask_size); 2: chunks (i sees j <= i of its own block of
+ *                             mask_size positions, counted from the start of the sequence); 0: every j <= i
+ *   score shaping             score = q . k * scale; then softcap * tanh(score / softcap) (softcap > 0); then minus slope_h * (i - j), slope_h =
+ *                             2^(-8 (h + 1) / heads) (dist_bias); queries times 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1) at position p
+ *   rotary variants           rot_pairs 1 turns neighbours (2i, 2i + 1) instead of (i, i + rot_dims / 2); every angle is divided by rot_factor (> 0)
+ *   shared keys and values    kv_share = 1 + j: the layer has no key / value projections and reads layer j's pool with its own queries and mask
+ *   wkv                       token shift (every projection reads h + (h_before - h) * mu of its own), a decay per key channel from a low-rank product
+ *                             (decay_rank), S <- diag(w) S + k v^T read with a bonus u for the current token, per-head unit norm, silu gate
+ *   gated delta rule          causal depth-wise convolutions of conv_taps taps and silu on q, k, v; unit q and k; S <- g S; S += k (beta (v - S^T k))^T;
+ *                             o = S^T q; per-head unit norm, a weight shared by the heads, silu gate
+ *   parallel mixer            left_scale * attention + right_scale * gated delta rule on the same input (the d_* fields size the right half)
+ *   dense gated feed-forward  down(silu(gate h) * (up h)) */
+typedef enum tgx_mixer { TGX_MIXER_LATENT_ATTENTION = 1, TGX_MIXER_ATTENTION = 2, TGX_MIXER_MLSTM = 3, TGX_MIXER_WKV = 4, TGX_MIXER_PARALLEL = 5 } tgx_mixer;
 typedef enum tgx_mlp { TGX_MLP_NONE = 0, TGX_MLP_MOE = 1, TGX_MLP_DENSE = 2 } tgx_mlp;
 
 typedef struct tgx_layer_desc {
@@ -144,10 +161,28 @@ typedef struct tgx_layer_desc {
   int32_t groups_keep; /* experts: groups whose members may be chosen                             */
   float router_scale;  /* experts: weights = scores * router_scale                                */
   int32_t shared_ff; /* experts: width of the shared expert (0: none)                             */
+  /* ABI 6 (zero for the kinds that do not read them) */
+  int32_t mask_kind; /* attention: 0 causal, 1 sliding window, 2 chunks                           */
+  int32_t mask_size; /* attention: window / chunk length in positions                             */
+  float softcap;     /* attention: soft cap of the scaled score (<= 0: none)                      */
+  int32_t dist_bias; /* attention: 1 = minus 2^(-8 (h + 1) / heads) * (i - j)                     */
+  float q_temp_coef; /* attention: query temperature (0: none) ...                                */
+  int32_t q_temp_every; /*         ... and its period in positions                               */
+  int32_t rot_pairs; /* attention: 1 = rotate neighbours (2i, 2i + 1)                             */
+  float rot_factor;  /* attention: angles are divided by this (<= 0: 1)                           */
+  int32_t kv_share;  /* attention: 1 + the layer whose keys and values this one reads (0: its own) */
+  int32_t decay_rank; /* wkv: inner size of the decay's low-rank product (0: from the tensors)    */
+  int32_t d_heads;   /* parallel: the gated delta rule's value heads ...                          */
+  int32_t d_kv_heads; /*          ... its query / key heads                                      */
+  int32_t d_dim;     /*           ... their size                                                 */
+  int32_t d_vdim;    /*           ... the value size per head                                    */
+  int32_t conv_taps; /*           ... taps of its input convolutions                             */
+  float left_scale;  /* parallel: weight of the attention half                                    */
+  float right_scale; /* parallel: weight of the gated delta rule                                  */
 } tgx_layer_desc;
 
 typedef struct tgx_stack_desc {
-  int32_t family;         /* tgx_family (TGX_FAMILY_ZAKUSUN, TGX_FAMILY_MODEPEL)                   */
+  int32_t family;         /* tgx_family (TGX_FAMILY_ZAKUSUN, TGX_FAMILY_MODEPEL, TGX_FAMILY_VITUDRA) */
   int32_t width;          /* residual width                                                        */
   int32_t layers;         /* entries of the tgx_layer_desc array                                   */
   int32_t vocab;
@@ -160,6 +195,7 @@ typedef struct tgx_stack_desc {
   float norm_eps;
   int32_t canon_taps;     /* taps of the input convolution (>= 1)                                  */
   float logit_scale;      /* logits = embed . norm(x) * logit_scale                                */
+  float residual_mult;    /* ABI 6, TGX_FAMILY_VITUDRA: the factor on what a layer adds to the stream */
 } tgx_stack_desc;
 
 /* SamplerConfig (src/engine/Sampler.h:13-22).  Greedy iff temperature<=0 && top_k<=0 &&
@@ -184,7 +220,9 @@ TGX_API int tgx_create(const tgx_model_desc* desc, int device_ordinal, tgx_ctx**
 /* The layered counterpart of tgx_create: `layers` holds desc->layers entries.  Checkpoint names (tgx_upload): "embed", "final.norm",
  * "l<i>.norm1|norm2|canon1|canon2|dwa", "l<i>.mix.q|dkv|dkv.norm|uk|uv|sink|g|o", "l<i>.mlp.router|router.b", "l<i>.mlp.e<j>.gate|up|down".
  * TGX_FAMILY_MODEPEL: "embed", "head", "final.norm", "l<i>.norm1|norm1b|norm2|norm2b", attention "l<i>.mix.q|k|v(.b)|vmix|g|o", mLSTM
- * "l<i>.mix.q|k|v|g|o|norm|i(.b)|f(.b)", dense "l<i>.mlp.up|down|act", experts "l<i>.mlp.router|correction|e<j>.gate|up|down|shared.gate|up|down|sg". */
+ * "l<i>.mix.q|k|v|g|o|norm|i(.b)|f(.b)", dense "l<i>.mlp.up|down|act", experts "l<i>.mlp.router|correction|e<j>.gate|up|down|shared.gate|up|down|sg".
+ * TGX_FAMILY_VITUDRA: "embed", "head", "final.norm", "l<i>.norm1", "l<i>.mlp.gate|up|down", attention "l<i>.mix.q|k|v|o" (no k, v with kv_share), wkv
+ * "l<i>.mix.mu.r|k|v|g|w", "l<i>.mix.r|k|v|g|w1|w2|w0|u|norm|o", parallel "l<i>.mix.left.q|k|v|o", "l<i>.mix.right.q|k|v(.conv)|b|a|A_log|dt_bias|g|norm|o". */
 TGX_API int tgx_create_stack(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int device_ordinal, tgx_ctx** out_ctx);
 
 /* == SafeTensors::loadInternal -> Storage::copyOnDevice for ONE named tensor

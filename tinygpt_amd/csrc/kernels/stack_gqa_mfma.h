@@ -28,13 +28,16 @@ struct GqaMfmaArgs {
   float* part; int nsplit, keys_per;   // keys_per: a multiple of 64
   int heads, kv_heads, dim, vdim, terms;
   float scale, sink; int has_sink;
+  int mask_kind, mask_size;            // MASK_* (stack_meta.h): a row sees the keys [first_key(position), position]
+  float softcap; int dist_bias;        // score shaping as in gqa_attn_kernel (softcap <= 0: none)
 };
 
 template <int DT, int ND, int NT, bool SPLIT>      // ND = dim / 64: 16-channel steps of a wave's share of the contraction; NT = ceil(vdim / 128): 32-column output tiles per wave
 __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaArgs a) {
   constexpr int RQ = 16 * ND, KS = ND;
   constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
-  const float qscale = a.scale * LOG2E;
+  const bool capped = a.softcap > 0.f;
+  const float qscale = capped ? a.scale : a.scale * LOG2E;      // a capped score is needed in natural units first
   __shared__ float s_part[4][32][65];
   __shared__ __attribute__((aligned(16))) bf16_t s_ph[32][72], s_pl[32][72];
   __shared__ float s_corr[32], s_l[32];
@@ -45,8 +48,9 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaA
   const int past = m.tok_pos[start];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, half = lane >> 5, l31 = lane & 31;
   const int kmax = past + min(r0 + 31, nrows - 1) / Gq + 1;      // keys of the tile's last row
-  int k0 = 0, k1 = kmax;
-  if (SPLIT) { k0 = min(kmax, (int)blockIdx.z * a.keys_per); k1 = min(kmax, k0 + a.keys_per); }
+  const int klo = first_key(past + r0 / Gq, a.mask_kind, a.mask_size) & ~63;      // the tile's first row sees the oldest key; whole key tiles
+  int k0 = klo, k1 = kmax;
+  if (SPLIT) { k0 = min(kmax, klo + (int)blockIdx.z * a.keys_per); k1 = min(kmax, k0 + a.keys_per); }
   const int page = 1 << m.page_shift, kd = a.kv_heads * a.dim, vd = a.kv_heads * a.vdim;
   const bf16_t* poolK = reinterpret_cast<const bf16_t*>(a.poolK) + (size_t)kvh * a.dim;
   const bf16_t* poolVT = reinterpret_cast<const bf16_t*>(a.poolVT);
@@ -79,6 +83,8 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaA
   const int sr = r0 + srow;
   const bool svalid = sr < nrows;
   const int skeys = svalid ? past + sr / Gq + 1 : 0;
+  const int slo = first_key(skeys - 1, a.mask_kind, a.mask_size);
+  const float slope2 = a.dist_bias && svalid ? distance_slope(kvh * Gq + sr % Gq, a.heads) * LOG2E : 0.f;
   const bool sinked = a.has_sink && svalid && (!SPLIT || blockIdx.z == 0);
   float m_s = sinked ? a.sink * LOG2E : -INFINITY, l_s = sinked ? 1.f : 0.f;      // the running maximum in base-2 units
 
@@ -131,8 +137,11 @@ __global__ __launch_bounds__(256) void gqa_attn_mfma_kernel(StepMeta m, GqaMfmaA
       float sv[8], tmax = -INFINITY;
 #pragma unroll
       for (int c = 0; c < 8; c++) {
-        const float v = s_part[0][srow][kq + c] + s_part[1][srow][kq + c] + s_part[2][srow][kq + c] + s_part[3][srow][kq + c];
-        sv[c] = (kt + kq + c < min(skeys, k1)) ? v : -INFINITY;
+        float v = s_part[0][srow][kq + c] + s_part[1][srow][kq + c] + s_part[2][srow][kq + c] + s_part[3][srow][kq + c];
+        const int key = kt + kq + c;
+        if (capped) v = a.softcap * tanhf(v / a.softcap) * LOG2E;
+        v = fmaf(-slope2, (float)(skeys - 1 - key), v);
+        sv[c] = (key >= slo && key < min(skeys, k1)) ? v : -INFINITY;
         tmax = fmaxf(tmax, sv[c]);
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 1, 64)); tmax = fmaxf(tmax, __shfl_xor(tmax, 2, 64)); tmax = fmaxf(tmax, __shfl_xor(tmax, 4, 64));

@@ -20,4 +20,12 @@ struct StepMeta {          // device arrays of one step (T tokens, S entries)
   int tbl_stride, page_shift, T, S;
 };
 
+// attention masks of the layered designs: the first key the query at position `pos` sees (its last is `pos`)
+enum { MASK_CAUSAL = 0, MASK_WINDOW = 1, MASK_CHUNK = 2 };
+__device__ __forceinline__ int first_key(int pos, int kind, int size) {
+  return kind == MASK_WINDOW ? max(0, pos - size + 1) : kind == MASK_CHUNK ? pos - pos % size : 0;
+}
+// the distance bias of head h of `heads`: scores lose slope * (i - j)
+__device__ __forceinline__ float distance_slope(int h, int heads) { return exp2f(-8.0f * (float)(h + 1) / (float)heads); }
+
 }  // namespace tgx

@@ -9,7 +9,7 @@
 //   gqa_attn_kernel         one (token, head) per workgroup against the pool: softmax with a constant sink, sigmoid gate on the output
 //   gqa_attn_kernel<.., SPLIT> + gqa_attn_merge_kernel   the same with a sequence's keys divided between workgroups
 //   mlstm_scan_kernel       the matrix-memory recurrence over an entry's tokens, state per slot in fp32
-//   mlstm_out_kernel        per-head RMS norm, learned scale and sigmoid gate of the recurrence's outputs
+//   head_norm_gate_kernel   per-head RMS norm, learned scale and sigmoid / silu gate of a recurrence's outputs
 //   router_group_kernel     softmax scores, correction, group limit, top-k, weights = scores * scale; the shared expert's gate
 #pragma once
 #include "stack.h"
@@ -100,33 +100,44 @@ __global__ __launch_bounds__(256) void poly_norm_kernel(float* z, const float* c
   }
 }
 
-// ---- rotary positions, value mixing and the pool append of one attention layer.  One workgroup per token.
-// proj row = [q (heads * dim) | k (kv_heads * dim) | v (kv_heads * vdim) | ...]; the pair (i, i + rot_dims / 2) of every q and k head turns by the
-// angle of (position, i), whose cosine and sine come from a host-made table.  q is rotated in place; k and v go to the pool in the storage dtype.
+// ---- rotary positions, query temperature, value mixing and the pool append of one attention layer.  One workgroup per token.
+// proj row = [q (heads * dim) | k (kv_heads * dim) | v (kv_heads * vdim) | ...]; a pair of channels of every q and k head turns by the angle of
+// (position, i), whose cosine and sine come from a host-made table: the pair is (i, i + rot_dims / 2), or the neighbours (2i, 2i + 1) with rot_pairs.
+// q is rotated in place (and multiplied by 1 + q_temp_coef * ln(floor((position + 1) / q_temp_every) + 1) where the design has a query temperature);
+// k and v go to the pool in the storage dtype.  A layer that reads another layer's keys and values has q alone in its row and no pool of its own.
 struct GqaAppendArgs {
   float* proj; long long ldp;
   int heads, kv_heads, dim, vdim, rot_dims;
   const float* cs;           // [positions][rot_dims / 2][2]
-  void* poolK;               // [pages][page_tokens][kv_heads * dim]
+  void* poolK;               // [pages][page_tokens][kv_heads * dim] (nullptr: nothing is appended, the row holds no k / v)
   void* poolV;               // [pages][page_tokens][kv_heads * vdim]
   void* poolVT;              // [pages][kv_heads * vdim][page_tokens]: the same values, token-contiguous per channel (nullptr: not kept)
   float* vfirst;             // [T][kv_heads * vdim] values of the first mixing layer for the step's tokens
   int vmode;                 // 0: no mixing; 1: this layer's values become vfirst; 2: v <- (1 - lam) v + lam vfirst
   const float* lam;
+  int rot_pairs;             // 1: neighbours turn together
+  float q_temp_coef; int q_temp_every;      // coef 0: no query temperature
 };
 template <int DT>
 __global__ __launch_bounds__(256) void gqa_append_kernel(StepMeta m, GqaAppendArgs a) {
   const int t = blockIdx.x, pos = m.tok_pos[t];
   float* row = a.proj + (size_t)t * a.ldp;
-  const int half = a.rot_dims >> 1, nh = a.heads + a.kv_heads;      // q heads and k heads are adjacent in the row: head index hd, offset hd * dim
+  const int half = a.rot_dims >> 1, nh = a.heads + (a.poolK ? a.kv_heads : 0);      // q heads and k heads are adjacent in the row: head index hd, offset hd * dim
   for (int i = threadIdx.x; i < nh * half; i += 256) {
     const int hd = i / half, p = i - hd * half;
     const float c = a.cs[((size_t)pos * half + p) * 2], s = a.cs[((size_t)pos * half + p) * 2 + 1];
-    float* u = row + (size_t)hd * a.dim + p;
-    const float x0 = u[0], x1 = u[half];
+    float* u = row + (size_t)hd * a.dim + (a.rot_pairs ? 2 * p : p);
+    const int other = a.rot_pairs ? 1 : half;
+    const float x0 = u[0], x1 = u[other];
     u[0] = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s));
-    u[half] = __fadd_rn(__fmul_rn(x1, c), __fmul_rn(x0, s));
+    u[other] = __fadd_rn(__fmul_rn(x1, c), __fmul_rn(x0, s));
   }
+  if (a.q_temp_coef != 0.f) {
+    __syncthreads();
+    const float f = fmaf(a.q_temp_coef, logf((float)((pos + 1) / a.q_temp_every) + 1.0f), 1.0f);
+    for (int c = threadIdx.x; c < a.heads * a.dim; c += 256) row[c] *= f;
+  }
+  if (!a.poolK) return;
   __syncthreads();
   const int page = m.tbl[(size_t)m.tok_row[t] * m.tbl_stride + (pos >> m.page_shift)];
   const size_t slot = ((size_t)page << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1));
@@ -150,6 +161,10 @@ __global__ __launch_bounds__(256) void gqa_append_kernel(StepMeta m, GqaAppendAr
 // ---- attention of one (token, head) per workgroup: the four waves take every fourth key, lanes hold dim / 64 key and vdim / 64 value channels.
 // Scores, softmax and the weighted value sum are fp32; the denominator also holds exp(sink) for a sink without a value (has_sink).  Every key, also
 // those of the step's own tokens, is read from the pool.  The output is multiplied by sigmoid(gate) where a gate is given.
+// The query at position i sees the keys [first_key(i), i]: all before it, a sliding window of mask_size positions, or its own block of mask_size
+// positions (blocks counted from position 0 of the sequence).  score = q . k * scale, then softcap * tanh(score / softcap), then minus
+// slope_h * (i - j), slope_h = 2^(-8 (h + 1) / heads), each where the layer has it.
+// (first_key and distance_slope: stack_meta.h)
 struct GqaAttnArgs {
   const float* q; long long ldq;       // head h of token t at q + t * ldq + h * dim
   const void* poolK; const void* poolV;
@@ -157,7 +172,9 @@ struct GqaAttnArgs {
   float* out; long long ldo;           // [T][heads * vdim]
   int heads, kv_heads, dim, vdim;
   float scale, sink; int has_sink;
-  float* part; int nsplit, keys_per;   // split form: records (m, l, acc[vdim]) per (token, head, split)
+  float* part; int nsplit, keys_per;   // split form: records (m, l, acc[vdim]) per (token, head, split); split z takes keys_per keys from first_key on
+  int mask_kind, mask_size;            // MASK_*
+  float softcap; int dist_bias;        // softcap <= 0: none
 };
 constexpr int GQA_MAX_RPL = 4;          // channels per lane: dim, vdim <= 256
 template <int DT, int RPL, bool SPLIT>
@@ -167,8 +184,9 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(StepMeta m, GqaAttnArgs a
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int row = m.tok_row[t], nkeys = m.tok_pos[t] + 1;
   const int kvh = h / (a.heads / a.kv_heads), kd = a.kv_heads * a.dim, vd = a.kv_heads * a.vdim;
-  int k0 = 0, k1 = nkeys;
-  if (SPLIT) { k0 = min(nkeys, (int)blockIdx.z * a.keys_per); k1 = min(nkeys, k0 + a.keys_per); }
+  int k0 = first_key(nkeys - 1, a.mask_kind, a.mask_size), k1 = nkeys;
+  if (SPLIT) { k0 = min(nkeys, k0 + (int)blockIdx.z * a.keys_per); k1 = min(nkeys, k0 + a.keys_per); }
+  const float slope = a.dist_bias ? distance_slope(h, a.heads) : 0.f;
   const float* q = a.q + (size_t)t * a.ldq + (size_t)h * a.dim;
   float qv[RPL], acc[RPL];
 #pragma unroll
@@ -191,6 +209,8 @@ __global__ __launch_bounds__(256) void gqa_attn_kernel(StepMeta m, GqaAttnArgs a
       vv[k] = c < a.vdim ? elem_to_f32<DT>(vr[c]) : 0.f;
     }
     s = wave_sum(s) * a.scale;
+    if (a.softcap > 0.f) s = a.softcap * tanhf(s / a.softcap);
+    s = fmaf(-slope, (float)(nkeys - 1 - j), s);
     const float mn = fmaxf(mx, s);
     const float corr = expf(mx - mn), p = expf(s - mn);      // mx = -inf on a wave's first key: corr = 0
     l = fmaf(l, corr, p);
@@ -261,7 +281,7 @@ __global__ __launch_bounds__(256) void gqa_attn_merge_kernel(GqaAttnArgs a) {
 //           column in registers and leaves its partial sums of S^T q and n . q (every wave computes the latter) per token in LDS
 //   out     the partial sums of the block's tokens are added up (over the row groups; over the wave for n . q) and divided
 // n and mx are double-buffered per slot (buffer `par` is read, `par ^ 1` written), because the workgroups of a head's other columns read them too.
-// The outputs leave un-normed (mlstm_out_kernel follows).
+// The outputs leave un-normed (head_norm_gate_kernel follows).
 struct MlstmArgs {
   const float* proj; long long ldp;     // [T][q | k | v | g | i | f]: q, k per head [dim]; v, g per head [vdim]; i, f per head: the log gates (the input product's epilogue has applied cap and log sigmoid)
   int heads, dim, vdim;
@@ -385,9 +405,10 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(StepMeta m, MlstmArgs a
   }
 }
 
-// out[t][h][c] = hs / sqrt(mean_c(hs^2) + eps) * w[h][c] * sigmoid(gate).  One wave per (token, head).
-struct MlstmOutArgs { const float* hs; long long ldh; const float* w; const float* gate; long long ldg; float* out; long long ldo; int vdim; float eps; };
-__global__ __launch_bounds__(64) void mlstm_out_kernel(MlstmOutArgs a) {
+// out[t][h][c] = hs / sqrt(mean_c(hs^2) + eps) * w[h * w_hstride + c] * gate, gate = sigmoid(z) or silu(z) of the pre-activation z (w_hstride 0: one
+// weight vector for all heads).  One wave per (token, head): the seam behind every recurrent mixer (mLSTM, wkv, gated delta rule).
+struct HeadNormGateArgs { const float* hs; long long ldh; const float* w; int w_hstride; const float* gate; long long ldg; int silu_gate; float* out; long long ldo; int vdim; float eps; };
+__global__ __launch_bounds__(64) void head_norm_gate_kernel(HeadNormGateArgs a) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float* r = a.hs + (size_t)t * a.ldh + (size_t)h * a.vdim;
   float ss = 0.f;
@@ -395,8 +416,8 @@ __global__ __launch_bounds__(64) void mlstm_out_kernel(MlstmOutArgs a) {
   ss = wave_sum(ss);
   const float rinv = 1.0f / sqrtf(ss / (float)a.vdim + a.eps);
   for (int c = lane; c < a.vdim; c += 64) {
-    const float g = a.gate[(size_t)t * a.ldg + (size_t)h * a.vdim + c];
-    a.out[(size_t)t * a.ldo + (size_t)h * a.vdim + c] = r[c] * rinv * a.w[(size_t)h * a.vdim + c] / (1.0f + expf(-g));
+    const float g = a.gate[(size_t)t * a.ldg + (size_t)h * a.vdim + c], sg = 1.0f / (1.0f + expf(-g));
+    a.out[(size_t)t * a.ldo + (size_t)h * a.vdim + c] = r[c] * rinv * a.w[(size_t)h * a.w_hstride + c] * (a.silu_gate ? g * sg : sg);
   }
 }
 

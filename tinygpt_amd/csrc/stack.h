@@ -37,9 +37,19 @@ struct StackLayerW {
   float* act = nullptr;
   // grouped-choice experts: w_router holds experts + identity rows and, with a shared expert, its gate row last; b_router is the correction
   ebyte *ws_gate = nullptr, *ws_up = nullptr, *ws_down = nullptr;      // shared expert
+  // parallel-sublayer designs (Vitudra).  norm1 holds the layer's norm weight (its distance from one); the gated feed-forward uses w_gate / w_up / w_down.
+  //   attention: w_in = [q | k | v] rows (q alone when the layer reads another layer's pool: kv_src, whose pool pointers it borrows)
+  //   wkv:       w_in = [r | k | v | g] (one product batched over the four token-shift mixes), w_w1 / w_w2 / w0 the decay's low-rank product, mu the five
+  //              mixing vectors, ubonus the current token's bonus, head_w the scale behind the per-head norm; mS the state, shift the slot's last row
+  //   parallel:  w_in = [left q | k | v | right q | k | v | b | a | g], w_o the left and w_o2 the right output projection; conv_w the right half's filters,
+  //              conv_state the tails of its raw projections, mS its state, head_w the weight all heads share
+  int kv_src = -1;
+  ebyte *w_o2 = nullptr, *w_w1 = nullptr, *w_w2 = nullptr;
+  float *mu = nullptr, *w0 = nullptr, *ubonus = nullptr, *conv_w = nullptr, *a_log = nullptr, *dt_bias = nullptr;
+  float* shift = nullptr;       // [2][slots][width]
 };
 
-struct RotTable { int dims; float base; float* cs; };      // cos / sin of (position, pair) [max_ctx][dims / 2][2], made on the host in double precision
+struct RotTable { int dims; float base; float factor; float* cs; };      // cos / sin of (position, pair) [max_ctx][dims / 2][2], angle = position * base^(-2 pair / dims) / factor, made on the host in double precision
 
 struct StackModel {
   tgx_stack_desc d{};
@@ -48,7 +58,10 @@ struct StackModel {
   float *final_norm = nullptr, *freq = nullptr;
   // what the family fixes (stack_create): the kind of norm and of layer wiring
   bool sandwich = false;               // scalar RMS norms before and after every sublayer, no convolutions, no depth average, no position vector, a separate head
-  ebyte* head = nullptr;               // [vocab][width] (sandwich designs; the others multiply by the embedding table)
+  bool joint = false;                  // one offset-weight RMS norm per layer; mixer and feed-forward read it side by side; x += residual_mult * (their sum); a separate head
+  float *mixed = nullptr, *lora = nullptr, *rec_in = nullptr;      // joint designs' step workspace: the token-shift mixes, the decay's inner product, the delta rule's inputs
+  int max_shift = 0, max_lora = 0, max_rec = 0;
+  ebyte* head = nullptr;               // [vocab][width] (sandwich and joint designs; the others multiply by the embedding table)
   float* norm_g = nullptr;             // [4 * layers + 1] norm numbers, the final norm's last
   std::vector<RotTable> rot;
   float *a2 = nullptr, *ytmp = nullptr, *ysh = nullptr, *sgw = nullptr, *vfirst = nullptr, *hs = nullptr;      // more step workspace

@@ -15,6 +15,7 @@
 #include "kernels/stack_attn_mfma.h"
 #include "kernels/stack_seq.h"
 #include "kernels/stack_gqa_mfma.h"
+#include "kernels/stack_rec.h"
 
 int upload_param_ext(tgx_ctx* c, ebyte* dst, const void* host, int64_t n, int src_dtype);      // abi.hip
 
@@ -170,7 +171,7 @@ int ensure_ws(tgx_ctx* c, int T) {
   auto fr = [](auto*& p) { if (p) (void)hipFree(p); p = nullptr; };
   fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw); fr(sm->yh); fr(sm->yd); fr(sm->xn); fr(sm->lg);
   fr(sm->sel); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->meta_dev); fr(sm->zr);
-  fr(sm->a2); fr(sm->ytmp); fr(sm->ysh); fr(sm->sgw); fr(sm->vfirst); fr(sm->hs);
+  fr(sm->a2); fr(sm->ytmp); fr(sm->ysh); fr(sm->sgw); fr(sm->vfirst); fr(sm->hs); fr(sm->mixed); fr(sm->lora); fr(sm->rec_in);
   if (sm->meta_host) { (void)hipHostFree(sm->meta_host); sm->meta_host = nullptr; }
   const int cap = std::max(T, 64);
   const size_t W = (size_t)sm->d.width, n = (size_t)cap;
@@ -178,6 +179,9 @@ int ensure_ws(tgx_ctx* c, int T) {
   if (sm->sandwich) {      // no layer results are kept; the seams need a second normed stream, a scratch row and the mixers' side buffers
     if ((rc = dev_alloc(c, &sm->a2, n * W)) || (rc = dev_alloc(c, &sm->ytmp, n * W)) || (rc = dev_alloc(c, &sm->ysh, n * W)) || (rc = dev_alloc(c, &sm->sgw, n)) ||
         (rc = dev_alloc(c, &sm->vfirst, n * (size_t)std::max(1, sm->max_kvv))) || (rc = dev_alloc(c, &sm->hs, n * (size_t)std::max(1, sm->max_hv)))) return rc;
+  } else if (sm->joint) {    // the recurrent mixers' side buffers: un-normed outputs, token-shift mixes, the decay's inner product, the delta rule's inputs
+    if ((rc = dev_alloc(c, &sm->hs, n * (size_t)std::max(1, sm->max_hv))) || (rc = dev_alloc(c, &sm->mixed, n * (size_t)std::max(1, sm->max_shift))) ||
+        (rc = dev_alloc(c, &sm->lora, n * (size_t)std::max(1, sm->max_lora))) || (rc = dev_alloc(c, &sm->rec_in, n * (size_t)std::max(1, sm->max_rec)))) return rc;
   } else if ((rc = dev_alloc(c, &sm->xs, (size_t)(sm->d.layers + 1) * n * W))) return rc;
   if ((rc = dev_alloc(c, &sm->x, n * W)) || (rc = dev_alloc(c, &sm->a, n * W)) ||
       (rc = dev_alloc(c, &sm->proj, n * (size_t)sm->max_in)) || (rc = dev_alloc(c, &sm->ql, n * (size_t)sm->max_hr)) || (rc = dev_alloc(c, &sm->lat, n * (size_t)sm->max_hr)) ||
@@ -285,7 +289,7 @@ int run_layers_latent(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys
     launch_gemm(c, g, tgx::SG_GATE, H);
     // x += o . w_o^T
     g = tgx::StackGemmArgs{};
-    g.A = sm->o; g.lda = vd; g.B = w.w_o; g.ldb = vd; g.C = sm->x; g.ldc = W; g.M = T; g.N = W; g.K = vd;
+    g.A = sm->o; g.lda = vd; g.B = w.w_o; g.ldb = vd; g.C = sm->x; g.ldc = W; g.M = T; g.N = W; g.K = vd; g.scale = 1.f;
     launch_gemm(c, g, tgx::SG_ADD, 1);
     int top = 0;
     if (ld.mlp == TGX_MLP_MOE) {
@@ -333,6 +337,82 @@ void launch_gqa_t(tgx_ctx* c, const tgx::StepMeta& m, const tgx::GqaAttnArgs& a,
   else hipLaunchKernelGGL((tgx::gqa_attn_kernel<DT, 4, SPLIT>), grid, dim3(256), lds, c->stream, m, a);
 }
 
+// One attention layer's work between its input and output products, for every design with grouped-query attention over a paged key / value pool: rotation /
+// query temperature / pool append, then the attention itself (matrix cores where the layer keeps a transposed value pool, lanes otherwise; a sequence's keys
+// divided between workgroups when the step is small and the span of visible keys long).  The projections' row is [q | k | v | ..] at `proj`.
+struct GqaSpec {
+  float* proj; long long ldp;
+  int heads, kv_heads, dim, vdim;
+  int rot_dims, rot_pairs; const float* cs;
+  ebyte *poolK, *poolV, *poolVT; bool append;      // append false: the pools belong to another layer, which has filled them for this step's tokens already
+  int vmode; const float* lam;
+  const float* gate; long long ldg;
+  float scale, sink; int has_sink;
+  int mask_kind, mask_size; float softcap; int dist_bias;
+  float q_temp_coef; int q_temp_every;
+  float* out; long long ldo;
+};
+int run_gqa_core(tgx_ctx* c, const tgx::StepMeta& m, const GqaSpec& sp, int T, int S, int max_keys, int max_count) {
+  StackModel* sm = c->stack;
+  const int H = sp.heads, G = sp.kv_heads;
+  tgx::GqaAppendArgs ap{};
+  ap.proj = sp.proj; ap.ldp = sp.ldp; ap.heads = H; ap.kv_heads = G; ap.dim = sp.dim; ap.vdim = sp.vdim; ap.rot_dims = sp.cs ? sp.rot_dims : 0; ap.rot_pairs = sp.rot_pairs;
+  ap.cs = sp.cs; ap.poolK = sp.append ? sp.poolK : nullptr; ap.poolV = sp.poolV; ap.poolVT = sp.poolVT; ap.vfirst = sm->vfirst; ap.vmode = sp.vmode; ap.lam = sp.lam;
+  ap.q_temp_coef = sp.q_temp_every > 0 ? sp.q_temp_coef : 0.f; ap.q_temp_every = sp.q_temp_every;
+  if (sp.append || ap.rot_dims > 0 || ap.q_temp_coef != 0.f) TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::gqa_append_kernel<DT>, dim3(T), dim3(256), 0, c->stream, m, ap))
+  // the longest run of keys any workgroup walks: everything before the token, or the mask's span (plus the matrix-core kernel's tile alignment)
+  const int span = sp.mask_kind == tgx::MASK_CAUSAL ? max_keys : std::min(max_keys, sp.mask_size + 96);
+  if (sp.poolVT && sm->attn_mfma) {
+    // rows = (token, query head of the group) pairs of an entry and a key / value head in tiles of 32; few tiles and a long context: the keys are divided
+    tgx::GqaMfmaArgs ma{};
+    ma.q = sp.proj; ma.ldq = sp.ldp; ma.poolK = sp.poolK; ma.poolVT = sp.poolVT; ma.gate = sp.gate; ma.ldg = sp.ldg; ma.out = sp.out; ma.ldo = sp.ldo;
+    ma.heads = H; ma.kv_heads = G; ma.dim = sp.dim; ma.vdim = sp.vdim; ma.terms = c->act16 ? 1 : 2; ma.scale = sp.scale; ma.sink = sp.sink; ma.has_sink = sp.has_sink;
+    ma.mask_kind = sp.mask_kind; ma.mask_size = sp.mask_size; ma.softcap = sp.softcap; ma.dist_bias = sp.dist_bias;
+    const int tiles = (max_count * (H / G) + 31) / 32;
+    const long long wgs = (long long)tiles * S * G;
+    int nsplit = 1;
+    if (span >= sm->attn_split_min_keys && wgs < c->num_cus) {
+      nsplit = (int)std::min<long long>(64, (2LL * c->num_cus) / wgs);
+      const int per = std::max(64, ((span + nsplit - 1) / nsplit + 63) / 64 * 64);      // whole key tiles
+      nsplit = (span + per - 1) / per;
+      ma.keys_per = per;
+    }
+    if (nsplit > 1) {
+      int rc = ensure_part(c, (size_t)T * H * nsplit * (size_t)(sp.vdim + 2));
+      if (rc) return rc;
+      ma.part = sm->part; ma.nsplit = nsplit;
+      launch_gqa_mfma(c, m, ma, dim3(tiles, S * G, nsplit), true);
+      tgx::GqaAttnArgs mg{};
+      mg.part = sm->part; mg.nsplit = nsplit; mg.heads = H; mg.vdim = sp.vdim; mg.gate = sp.gate; mg.ldg = sp.ldg; mg.out = sp.out; mg.ldo = sp.ldo;
+      hipLaunchKernelGGL(tgx::gqa_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, mg);
+    } else {
+      launch_gqa_mfma(c, m, ma, dim3(tiles, S * G), false);
+    }
+    return TGX_OK;
+  }
+  tgx::GqaAttnArgs aa{};
+  aa.q = sp.proj; aa.ldq = sp.ldp; aa.poolK = sp.poolK; aa.poolV = sp.poolV; aa.gate = sp.gate; aa.ldg = sp.ldg; aa.out = sp.out; aa.ldo = sp.ldo;
+  aa.heads = H; aa.kv_heads = G; aa.dim = sp.dim; aa.vdim = sp.vdim; aa.scale = sp.scale; aa.sink = sp.sink; aa.has_sink = sp.has_sink;
+  aa.mask_kind = sp.mask_kind; aa.mask_size = sp.mask_size; aa.softcap = sp.softcap; aa.dist_bias = sp.dist_bias;
+  int nsplit = 1;
+  if (span >= sm->attn_split_min_keys && (long long)T * H < 2LL * c->num_cus) {      // few (token, head) pairs and a long context: the keys are divided between workgroups
+    nsplit = (int)std::min<long long>(64, (4LL * c->num_cus) / ((long long)T * H));
+    const int per = std::max(256, ((span + nsplit - 1) / nsplit + 63) / 64 * 64);
+    nsplit = (span + per - 1) / per;
+    aa.keys_per = per;
+  }
+  if (nsplit > 1) {
+    int rc = ensure_part(c, (size_t)T * H * nsplit * (size_t)(sp.vdim + 2));
+    if (rc) return rc;
+    aa.part = sm->part; aa.nsplit = nsplit;
+    TGX_DT_SWITCH(c->dt, (launch_gqa_t<DT, true>(c, m, aa, dim3(T, H, nsplit))))
+    hipLaunchKernelGGL(tgx::gqa_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, aa);
+  } else {
+    TGX_DT_SWITCH(c->dt, (launch_gqa_t<DT, false>(c, m, aa, dim3(T, H))))
+  }
+  return TGX_OK;
+}
+
 int run_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const float* hin, int T, int S, int max_keys, int max_count) {
   StackModel* sm = c->stack;
   const tgx_layer_desc& ld = w.d;
@@ -341,56 +421,12 @@ int run_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const floa
   tgx::StackGemmArgs g{};
   g.A = hin; g.lda = W; g.B = w.w_in; g.ldb = W; g.C = sm->proj; g.ldc = nin; g.M = T; g.N = nin; g.K = W; g.scale = 1.f; g.bias = w.b_in;
   launch_gemm(c, g, tgx::SG_STORE, 1);
-  tgx::GqaAppendArgs ap{};
-  ap.proj = sm->proj; ap.ldp = nin; ap.heads = H; ap.kv_heads = G; ap.dim = ld.dim; ap.vdim = ld.vdim; ap.rot_dims = ld.rot_dims;
-  ap.cs = w.rot >= 0 ? sm->rot[(size_t)w.rot].cs : nullptr; ap.poolK = w.pool; ap.poolV = w.poolV; ap.poolVT = w.poolVT; ap.vfirst = sm->vfirst; ap.vmode = w.vmode; ap.lam = w.vmix;
-  TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::gqa_append_kernel<DT>, dim3(T), dim3(256), 0, c->stream, m, ap))
-  if (w.poolVT && sm->attn_mfma) {
-    // rows = (token, query head of the group) pairs of an entry and a key / value head in tiles of 32; few tiles and a long context: the keys are divided
-    tgx::GqaMfmaArgs ma{};
-    ma.q = sm->proj; ma.ldq = nin; ma.poolK = w.pool; ma.poolVT = w.poolVT; ma.gate = sm->proj + qd + kd + kvv; ma.ldg = nin; ma.out = sm->o; ma.ldo = vd;
-    ma.heads = H; ma.kv_heads = G; ma.dim = ld.dim; ma.vdim = ld.vdim; ma.terms = c->act16 ? 1 : 2; ma.scale = ld.scale; ma.sink = 0.f; ma.has_sink = 1;
-    const int tiles = (max_count * (H / G) + 31) / 32;
-    const long long wgs = (long long)tiles * S * G;
-    int nsplit = 1;
-    if (max_keys >= sm->attn_split_min_keys && wgs < c->num_cus) {
-      nsplit = (int)std::min<long long>(64, (2LL * c->num_cus) / wgs);
-      const int per = std::max(64, ((max_keys + nsplit - 1) / nsplit + 63) / 64 * 64);      // whole key tiles
-      nsplit = (max_keys + per - 1) / per;
-      ma.keys_per = per;
-    }
-    if (nsplit > 1) {
-      int rc = ensure_part(c, (size_t)T * H * nsplit * (size_t)(ld.vdim + 2));
-      if (rc) return rc;
-      ma.part = sm->part; ma.nsplit = nsplit;
-      launch_gqa_mfma(c, m, ma, dim3(tiles, S * G, nsplit), true);
-      tgx::GqaAttnArgs mg{};
-      mg.part = sm->part; mg.nsplit = nsplit; mg.heads = H; mg.vdim = ld.vdim; mg.gate = ma.gate; mg.ldg = nin; mg.out = sm->o; mg.ldo = vd;
-      hipLaunchKernelGGL(tgx::gqa_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, mg);
-    } else {
-      launch_gqa_mfma(c, m, ma, dim3(tiles, S * G), false);
-    }
-  } else {
-  tgx::GqaAttnArgs aa{};
-  aa.q = sm->proj; aa.ldq = nin; aa.poolK = w.pool; aa.poolV = w.poolV; aa.gate = sm->proj + qd + kd + kvv; aa.ldg = nin; aa.out = sm->o; aa.ldo = vd;
-  aa.heads = H; aa.kv_heads = G; aa.dim = ld.dim; aa.vdim = ld.vdim; aa.scale = ld.scale; aa.sink = 0.f; aa.has_sink = 1;
-  int nsplit = 1;
-  if (max_keys >= sm->attn_split_min_keys && (long long)T * H < 2LL * c->num_cus) {      // few (token, head) pairs and a long context: the keys are divided between workgroups
-    nsplit = (int)std::min<long long>(64, (4LL * c->num_cus) / ((long long)T * H));
-    const int per = std::max(256, ((max_keys + nsplit - 1) / nsplit + 63) / 64 * 64);
-    nsplit = (max_keys + per - 1) / per;
-    aa.keys_per = per;
-  }
-  if (nsplit > 1) {
-    int rc = ensure_part(c, (size_t)T * H * nsplit * (size_t)(ld.vdim + 2));
-    if (rc) return rc;
-    aa.part = sm->part; aa.nsplit = nsplit;
-    TGX_DT_SWITCH(c->dt, (launch_gqa_t<DT, true>(c, m, aa, dim3(T, H, nsplit))))
-    hipLaunchKernelGGL(tgx::gqa_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, aa);
-  } else {
-    TGX_DT_SWITCH(c->dt, (launch_gqa_t<DT, false>(c, m, aa, dim3(T, H))))
-  }
-  }
+  GqaSpec sp{};
+  sp.proj = sm->proj; sp.ldp = nin; sp.heads = H; sp.kv_heads = G; sp.dim = ld.dim; sp.vdim = ld.vdim; sp.rot_dims = ld.rot_dims;
+  sp.cs = w.rot >= 0 ? sm->rot[(size_t)w.rot].cs : nullptr; sp.poolK = w.pool; sp.poolV = w.poolV; sp.poolVT = w.poolVT; sp.append = true; sp.vmode = w.vmode; sp.lam = w.vmix;
+  sp.gate = sm->proj + qd + kd + kvv; sp.ldg = nin; sp.scale = ld.scale; sp.sink = 0.f; sp.has_sink = 1; sp.out = sm->o; sp.ldo = vd;
+  int rc = run_gqa_core(c, m, sp, T, S, max_keys, max_count);
+  if (rc) return rc;
   // y = o . w_o^T
   g = tgx::StackGemmArgs{};
   g.A = sm->o; g.lda = vd; g.B = w.w_o; g.ldb = vd; g.C = sm->yd; g.ldc = W; g.M = T; g.N = W; g.K = vd; g.scale = 1.f;
@@ -428,9 +464,9 @@ int run_mlstm(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const float* h
     else if (dper <= 64) hipLaunchKernelGGL((tgx::mlstm_scan_kernel<64, 16>), grid, dim3(256), 0, c->stream, m, ma);
     else hipLaunchKernelGGL((tgx::mlstm_scan_kernel<128, 16>), grid, dim3(256), 0, c->stream, m, ma);
   }
-  tgx::MlstmOutArgs oa{};
-  oa.hs = sm->hs; oa.ldh = vd; oa.w = w.head_w; oa.gate = sm->proj + 2 * qd + vd; oa.ldg = nin; oa.out = sm->o; oa.ldo = vd; oa.vdim = ld.vdim; oa.eps = sm->d.norm_eps;
-  hipLaunchKernelGGL(tgx::mlstm_out_kernel, dim3(T, H), dim3(64), 0, c->stream, oa);
+  tgx::HeadNormGateArgs oa{};
+  oa.hs = sm->hs; oa.ldh = vd; oa.w = w.head_w; oa.w_hstride = ld.vdim; oa.gate = sm->proj + 2 * qd + vd; oa.ldg = nin; oa.out = sm->o; oa.ldo = vd; oa.vdim = ld.vdim; oa.eps = sm->d.norm_eps;
+  hipLaunchKernelGGL(tgx::head_norm_gate_kernel, dim3(T, H), dim3(64), 0, c->stream, oa);
   g = tgx::StackGemmArgs{};
   g.A = sm->o; g.lda = vd; g.B = w.w_o; g.ldb = vd; g.C = sm->yd; g.ldc = W; g.M = T; g.N = W; g.K = vd; g.scale = 1.f;
   launch_gemm(c, g, tgx::SG_STORE, 1);
@@ -520,7 +556,138 @@ int run_layers_sandwich(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_ke
   return TGX_OK;
 }
 
+// ---- parallel-sublayer designs (Vitudra): per layer  h = norm(x);  x += mult * (mixer(h) + ff(h)).  Every sublayer's last product adds its share to the
+// stream in its epilogue (mult, and the half's weight in a parallel mixer, as the product's scale), so no combine launch is needed.
+void add_to_stream(tgx_ctx* c, const float* A, int K, const ebyte* Wm, int T, float scale) {
+  StackModel* sm = c->stack;
+  tgx::StackGemmArgs g{};
+  g.A = A; g.lda = K; g.B = Wm; g.ldb = K; g.C = sm->x; g.ldc = sm->d.width; g.M = T; g.N = sm->d.width; g.K = K; g.scale = scale;
+  launch_gemm(c, g, tgx::SG_ADD, 1);
+}
+
+void launch_rec_scan(tgx_ctx* c, const tgx::StepMeta& m, const tgx::RecScanArgs& a, int kind, int S) {
+  const dim3 grid(S, a.heads, (a.vdim + 63) / 64);
+  const int dper = (a.dim + 3) / 4;
+  auto go = [&](auto K) {
+    constexpr int KIND = decltype(K)::value;
+    if (dper <= 8) hipLaunchKernelGGL((tgx::rec_scan_kernel<8, KIND>), grid, dim3(256), 0, c->stream, m, a);
+    else if (dper <= 16) hipLaunchKernelGGL((tgx::rec_scan_kernel<16, KIND>), grid, dim3(256), 0, c->stream, m, a);
+    else if (dper <= 32) hipLaunchKernelGGL((tgx::rec_scan_kernel<32, KIND>), grid, dim3(256), 0, c->stream, m, a);
+    else hipLaunchKernelGGL((tgx::rec_scan_kernel<64, KIND>), grid, dim3(256), 0, c->stream, m, a);
+  };
+  if (kind == tgx::REC_WKV) go(std::integral_constant<int, tgx::REC_WKV>{}); else go(std::integral_constant<int, tgx::REC_DELTA>{});
+}
+
+int run_joint_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, int T, int S, int max_keys, int max_count) {
+  StackModel* sm = c->stack;
+  const tgx_layer_desc& ld = w.d;
+  const bool shared = w.kv_src >= 0;
+  const int W = sm->d.width, H = ld.heads, G = ld.kv_heads, qd = H * ld.dim, vd = H * ld.vdim, nin = qd + (shared ? 0 : G * (ld.dim + ld.vdim));
+  tgx::StackGemmArgs g{};
+  g.A = sm->a; g.lda = W; g.B = w.w_in; g.ldb = W; g.C = sm->proj; g.ldc = nin; g.M = T; g.N = nin; g.K = W; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  GqaSpec sp{};
+  sp.proj = sm->proj; sp.ldp = nin; sp.heads = H; sp.kv_heads = G; sp.dim = ld.dim; sp.vdim = ld.vdim; sp.rot_dims = ld.rot_dims; sp.rot_pairs = ld.rot_pairs;
+  sp.cs = w.rot >= 0 ? sm->rot[(size_t)w.rot].cs : nullptr; sp.poolK = w.pool; sp.poolV = w.poolV; sp.poolVT = w.poolVT; sp.append = !shared;
+  sp.scale = ld.scale; sp.mask_kind = ld.mask_kind; sp.mask_size = ld.mask_size; sp.softcap = ld.softcap; sp.dist_bias = ld.dist_bias;
+  sp.q_temp_coef = ld.q_temp_coef; sp.q_temp_every = ld.q_temp_every; sp.out = sm->o; sp.ldo = vd;
+  int rc = run_gqa_core(c, m, sp, T, S, max_keys, max_count);
+  if (rc) return rc;
+  add_to_stream(c, sm->o, vd, w.w_o, T, sm->d.residual_mult);
+  return TGX_OK;
+}
+
+void run_wkv(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, int T, int S) {
+  StackModel* sm = c->stack;
+  const tgx_layer_desc& ld = w.d;
+  const int W = sm->d.width, H = ld.heads, HD = H * ld.dim, R = ld.decay_rank;
+  tgx::TokenShiftArgs ts{};
+  ts.h = sm->a; ts.mu = w.mu; ts.out = sm->mixed; ts.state = w.shift; ts.state_buf = (size_t)sm->d.max_seqs * W; ts.W = W; ts.n = 5;
+  hipLaunchKernelGGL(tgx::token_shift_kernel, dim3(T), dim3(256), 0, c->stream, m, ts);
+  // proj row = [r | k | v | g | w]: the first four as one product batched over their mixes, the decay through its low-rank pair
+  tgx::StackGemmArgs g{};
+  g.A = sm->mixed; g.lda = 5LL * W; g.a_zoff = W; g.B = w.w_in; g.ldb = W; g.b_zstride = (long long)HD * W; g.C = sm->proj; g.ldc = 5LL * HD; g.c_zoff = HD;
+  g.M = T; g.N = HD; g.K = W; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 4);
+  g = tgx::StackGemmArgs{};
+  g.A = sm->mixed + 4 * (size_t)W; g.lda = 5LL * W; g.B = w.w_w1; g.ldb = W; g.C = sm->lora; g.ldc = R; g.M = T; g.N = R; g.K = W; g.scale = 1.f; g.act = tgx::SG_ACT_TANH;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  g = tgx::StackGemmArgs{};
+  g.A = sm->lora; g.lda = R; g.B = w.w_w2; g.ldb = R; g.C = sm->proj + 4 * (size_t)HD; g.ldc = 5LL * HD; g.M = T; g.N = HD; g.K = R; g.scale = 1.f; g.bias = w.w0; g.act = tgx::SG_ACT_DECAY;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  tgx::RecScanArgs ra{};
+  ra.a = sm->proj; ra.lda = 5LL * HD; ra.k = sm->proj + HD; ra.ldk = 5LL * HD; ra.v = sm->proj + 2 * (size_t)HD; ra.ldv = 5LL * HD; ra.w = sm->proj + 4 * (size_t)HD; ra.ldw = 5LL * HD;
+  ra.u = w.ubonus; ra.S = w.mS; ra.out = sm->hs; ra.ldo = HD; ra.heads = H; ra.kv_heads = H; ra.dim = ld.dim; ra.vdim = ld.dim;
+  launch_rec_scan(c, m, ra, tgx::REC_WKV, S);
+  tgx::HeadNormGateArgs oa{};
+  oa.hs = sm->hs; oa.ldh = HD; oa.w = w.head_w; oa.w_hstride = ld.dim; oa.gate = sm->proj + 3 * (size_t)HD; oa.ldg = 5LL * HD; oa.silu_gate = 1; oa.out = sm->o; oa.ldo = HD; oa.vdim = ld.dim;
+  oa.eps = sm->d.norm_eps;
+  hipLaunchKernelGGL(tgx::head_norm_gate_kernel, dim3(T, H), dim3(64), 0, c->stream, oa);
+  add_to_stream(c, sm->o, HD, w.w_o, T, sm->d.residual_mult);
+}
+
+int run_parallel(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, int T, int S, int max_keys, int max_count) {
+  StackModel* sm = c->stack;
+  const tgx_layer_desc& ld = w.d;
+  const int W = sm->d.width, H = ld.heads, G = ld.kv_heads, lq = H * ld.dim, lkv = G * (ld.dim + ld.vdim), lvd = H * ld.vdim;
+  const int rH = ld.d_heads, rG = ld.d_kv_heads, rGD = rG * ld.d_dim, rvd = rH * ld.d_vdim, rC = 2 * rGD + rvd, nin = lq + lkv + rC + 2 * rH + rvd;
+  // [left q | k | v | right q | k | v | b | a | g] = h . w_in^T: both halves read the same input
+  tgx::StackGemmArgs g{};
+  g.A = sm->a; g.lda = W; g.B = w.w_in; g.ldb = W; g.C = sm->proj; g.ldc = nin; g.M = T; g.N = nin; g.K = W; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  GqaSpec sp{};
+  sp.proj = sm->proj; sp.ldp = nin; sp.heads = H; sp.kv_heads = G; sp.dim = ld.dim; sp.vdim = ld.vdim; sp.rot_dims = ld.rot_dims; sp.rot_pairs = ld.rot_pairs;
+  sp.cs = w.rot >= 0 ? sm->rot[(size_t)w.rot].cs : nullptr; sp.poolK = w.pool; sp.poolV = w.poolV; sp.poolVT = w.poolVT; sp.append = true;
+  sp.scale = ld.scale; sp.mask_kind = ld.mask_kind; sp.mask_size = ld.mask_size; sp.softcap = ld.softcap; sp.dist_bias = ld.dist_bias;
+  sp.q_temp_coef = ld.q_temp_coef; sp.q_temp_every = ld.q_temp_every; sp.out = sm->o; sp.ldo = lvd;
+  int rc = run_gqa_core(c, m, sp, T, S, max_keys, max_count);
+  if (rc) return rc;
+  add_to_stream(c, sm->o, lvd, w.w_o, T, sm->d.residual_mult * ld.left_scale);
+  // the right half: rec_in row = [q | k | v | beta | decay]
+  const int ldr = rC + 2 * rH, nb = ld.conv_taps - 1;
+  tgx::DeltaPrepArgs dp{};
+  dp.proj = sm->proj; dp.ldp = nin; dp.col0 = lq + lkv; dp.cw = w.conv_w; dp.a_log = w.a_log; dp.dt_bias = w.dt_bias; dp.out = sm->rec_in; dp.ldo = ldr;
+  dp.state = nb > 0 ? w.conv_state : nullptr; dp.state_buf = (size_t)sm->d.max_seqs * nb * rC; dp.heads = rH; dp.kv_heads = rG; dp.dim = ld.d_dim; dp.vdim = ld.d_vdim; dp.taps = ld.conv_taps;
+  dp.q_scale = 1.0f / sqrtf((float)ld.d_dim); dp.unit_eps = 1e-6f;
+  hipLaunchKernelGGL(tgx::delta_prep_kernel, dim3(T), dim3(256), (size_t)rC * 4, c->stream, m, dp);
+  tgx::RecScanArgs ra{};
+  ra.a = sm->rec_in; ra.lda = ldr; ra.k = sm->rec_in + rGD; ra.ldk = ldr; ra.v = sm->rec_in + 2 * (size_t)rGD; ra.ldv = ldr;
+  ra.beta = sm->rec_in + rC; ra.g = sm->rec_in + rC + rH; ra.ldg = ldr; ra.S = w.mS; ra.out = sm->hs; ra.ldo = rvd; ra.heads = rH; ra.kv_heads = rG; ra.dim = ld.d_dim; ra.vdim = ld.d_vdim;
+  launch_rec_scan(c, m, ra, tgx::REC_DELTA, S);
+  tgx::HeadNormGateArgs oa{};
+  oa.hs = sm->hs; oa.ldh = rvd; oa.w = w.head_w; oa.w_hstride = 0; oa.gate = sm->proj + lq + lkv + rC + 2 * rH; oa.ldg = nin; oa.silu_gate = 1; oa.out = sm->o; oa.ldo = rvd; oa.vdim = ld.d_vdim;
+  oa.eps = sm->d.norm_eps;
+  hipLaunchKernelGGL(tgx::head_norm_gate_kernel, dim3(T, rH), dim3(64), 0, c->stream, oa);
+  add_to_stream(c, sm->o, rvd, w.w_o2, T, sm->d.residual_mult * ld.right_scale);
+  return TGX_OK;
+}
+
+int run_layers_joint(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int max_count) {
+  StackModel* sm = c->stack;
+  const tgx::StepMeta m = step_meta(sm, mp, T, S);
+  const int W = sm->d.width;
+  TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::embed_rows_kernel<DT>, dim3(T), dim3(256), 0, c->stream, m, reinterpret_cast<const tgx::elem_t<DT>*>(c->embed), sm->x, W))
+  for (int li = 0; li < sm->d.layers; li++) {
+    StackLayerW& w = sm->L[(size_t)li];
+    const tgx_layer_desc& ld = w.d;
+    hipLaunchKernelGGL(tgx::offset_norm_kernel, dim3(T), dim3(256), 0, c->stream, sm->x, nullptr, w.norm1, 1.0f, sm->a, W, sm->d.norm_eps);
+    int rc = TGX_OK;
+    if (ld.mixer == TGX_MIXER_ATTENTION) rc = run_joint_attention(c, m, w, T, S, max_keys, max_count);
+    else if (ld.mixer == TGX_MIXER_WKV) run_wkv(c, m, w, T, S);
+    else rc = run_parallel(c, m, w, T, S, max_keys, max_count);
+    if (rc) return rc;
+    if (ld.mlp == TGX_MLP_DENSE) {      // x += mult * down(silu(gate h) * (up h))
+      tgx::StackGemmArgs g{};
+      g.A = sm->a; g.lda = W; g.B = w.w_gate; g.B2 = w.w_up; g.ldb = W; g.C = sm->yh; g.ldc = ld.ff; g.M = T; g.N = ld.ff; g.K = W;
+      launch_gemm(c, g, tgx::SG_SILU_MUL, 1);
+      add_to_stream(c, sm->yh, ld.ff, w.w_down, T, sm->d.residual_mult);
+    }
+  }
+  return TGX_OK;
+}
+
 int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int max_count) {
+  if (c->stack->joint) return run_layers_joint(c, mp, T, S, max_keys, max_count);
   return c->stack->sandwich ? run_layers_sandwich(c, mp, T, S, max_keys, max_count) : run_layers_latent(c, mp, T, S, max_keys, max_count);
 }
 
@@ -528,7 +695,8 @@ int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int m
 void run_logits(tgx_ctx* c, const int* want_dev, int nw, float* C, const int* c_rows) {
   StackModel* sm = c->stack;
   const int W = sm->d.width, V = sm->d.vocab;
-  if (sm->sandwich) hipLaunchKernelGGL(tgx::scalar_norm_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->norm_g + 4 * (size_t)sm->d.layers, sm->xn, W, sm->d.norm_eps);
+  if (sm->joint) hipLaunchKernelGGL(tgx::offset_norm_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->final_norm, 1.0f, sm->xn, W, sm->d.norm_eps);
+  else if (sm->sandwich) hipLaunchKernelGGL(tgx::scalar_norm_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->norm_g + 4 * (size_t)sm->d.layers, sm->xn, W, sm->d.norm_eps);
   else hipLaunchKernelGGL(tgx::final_norm_rows_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->final_norm, sm->xn, W, sm->d.norm_groups, sm->d.norm_eps);
   tgx::StackGemmArgs g{};
   g.A = sm->xn; g.lda = W; g.B = sm->head ? sm->head : c->embed; g.ldb = W; g.C = C; g.ldc = V; g.c_rows = c_rows; g.M = nw; g.N = V; g.K = W; g.scale = sm->d.logit_scale;
@@ -610,7 +778,7 @@ int create_sandwich_layers(tgx_ctx* c, const tgx_layer_desc* layers) {
       }
       if (l.rot_dims > 0) {
         for (size_t r = 0; r < sm->rot.size(); r++) if (sm->rot[r].dims == l.rot_dims && sm->rot[r].base == l.rot_base) w.rot = (int)r;
-        if (w.rot < 0) { w.rot = (int)sm->rot.size(); sm->rot.push_back(RotTable{l.rot_dims, l.rot_base, nullptr}); }
+        if (w.rot < 0) { w.rot = (int)sm->rot.size(); sm->rot.push_back(RotTable{l.rot_dims, l.rot_base, 1.f, nullptr}); }
       }
       sm->max_kvv = std::max(sm->max_kvv, (int)kvv);
     } else {
@@ -733,6 +901,152 @@ int upload_sandwich(tgx_ctx* c, const char* name, const void* host, const int64_
   return set_err(c, TGX_ERR_NAME, "Unexpected key: %s", name);
 }
 
+// parameter storage of a parallel-sublayer design (Vitudra): per layer the norm weight, the mixer of its kind and the gated feed-forward
+int create_joint_layers(tgx_ctx* c, const tgx_layer_desc* layers) {
+  StackModel* sm = c->stack;
+  const tgx_stack_desc& d = sm->d;
+  const size_t W = (size_t)d.width, es = c->esz;
+  int rc;
+  if ((rc = dev_alloc(c, &sm->head, (size_t)d.vocab * W * es))) return rc;
+  sm->missing.insert("head");
+  sm->max_top = 1; sm->max_E = 1; sm->max_ff = 1;      // the feed-forward's hidden row uses the expert buffers with one row per token
+  auto need = [&](const std::string& p, std::initializer_list<const char*> names) { for (const char* n : names) sm->missing.insert(p + n); };
+  for (int i = 0; i < d.layers; i++) {
+    StackLayerW& w = sm->L[(size_t)i];
+    w.d = layers[i];
+    const tgx_layer_desc& l = w.d;
+    const std::string p = "l" + std::to_string(i) + ".";
+    if ((rc = dev_alloc(c, &w.norm1, W))) return rc;
+    need(p, {"norm1"});
+    auto rotation = [&]() {
+      if (l.rot_dims <= 0) return;
+      const float factor = l.rot_factor > 0.f ? l.rot_factor : 1.f;
+      for (size_t r = 0; r < sm->rot.size(); r++) if (sm->rot[r].dims == l.rot_dims && sm->rot[r].base == l.rot_base && sm->rot[r].factor == factor) w.rot = (int)r;
+      if (w.rot < 0) { w.rot = (int)sm->rot.size(); sm->rot.push_back(RotTable{l.rot_dims, l.rot_base, factor, nullptr}); }
+    };
+    if (l.mixer == TGX_MIXER_ATTENTION) {
+      w.kv_src = l.kv_share - 1;
+      const size_t qd = (size_t)l.heads * l.dim, vd = (size_t)l.heads * l.vdim, nin = qd + (w.kv_src >= 0 ? 0 : (size_t)l.kv_heads * (l.dim + l.vdim));
+      if ((rc = dev_alloc(c, &w.w_in, nin * W * es)) || (rc = dev_alloc(c, &w.w_o, W * vd * es))) return rc;
+      need(p, {"mix.q", "mix.o"});
+      if (w.kv_src < 0) need(p, {"mix.k", "mix.v"});
+      rotation();
+      sm->max_in = std::max(sm->max_in, (int)nin); sm->max_hv = std::max(sm->max_hv, (int)vd);
+    } else if (l.mixer == TGX_MIXER_WKV) {
+      const size_t HD = (size_t)l.heads * l.dim;
+      if ((rc = dev_alloc(c, &w.w_in, 4 * HD * W * es)) || (rc = dev_alloc(c, &w.w_o, W * HD * es)) || (rc = dev_alloc(c, &w.mu, 5 * W)) || (rc = dev_alloc(c, &w.w0, HD)) ||
+          (rc = dev_alloc(c, &w.ubonus, HD)) || (rc = dev_alloc(c, &w.head_w, HD))) return rc;
+      if (l.decay_rank > 0 && ((rc = dev_alloc(c, &w.w_w1, (size_t)l.decay_rank * W * es)) || (rc = dev_alloc(c, &w.w_w2, HD * l.decay_rank * es)))) return rc;
+      need(p, {"mix.mu.r", "mix.mu.k", "mix.mu.v", "mix.mu.g", "mix.mu.w", "mix.r", "mix.k", "mix.v", "mix.g", "mix.w1", "mix.w2", "mix.w0", "mix.u", "mix.norm", "mix.o"});
+      sm->max_in = std::max(sm->max_in, (int)(5 * HD)); sm->max_hv = std::max(sm->max_hv, (int)HD); sm->max_shift = std::max(sm->max_shift, (int)(5 * W));
+      sm->max_lora = std::max(sm->max_lora, l.decay_rank);
+    } else {
+      const size_t lq = (size_t)l.heads * l.dim, lkv = (size_t)l.kv_heads * (l.dim + l.vdim), lvd = (size_t)l.heads * l.vdim;
+      const size_t rGD = (size_t)l.d_kv_heads * l.d_dim, rvd = (size_t)l.d_heads * l.d_vdim, rC = 2 * rGD + rvd, nin = lq + lkv + rC + 2 * (size_t)l.d_heads + rvd;
+      if ((rc = dev_alloc(c, &w.w_in, nin * W * es)) || (rc = dev_alloc(c, &w.w_o, W * lvd * es)) || (rc = dev_alloc(c, &w.w_o2, W * rvd * es)) ||
+          (rc = dev_alloc(c, &w.conv_w, rC * (size_t)l.conv_taps)) || (rc = dev_alloc(c, &w.a_log, (size_t)l.d_heads)) || (rc = dev_alloc(c, &w.dt_bias, (size_t)l.d_heads)) ||
+          (rc = dev_alloc(c, &w.head_w, (size_t)l.d_vdim))) return rc;
+      need(p, {"mix.left.q", "mix.left.k", "mix.left.v", "mix.left.o", "mix.right.q", "mix.right.k", "mix.right.v", "mix.right.q.conv", "mix.right.k.conv", "mix.right.v.conv",
+               "mix.right.b", "mix.right.a", "mix.right.A_log", "mix.right.dt_bias", "mix.right.g", "mix.right.norm", "mix.right.o"});
+      rotation();
+      sm->max_in = std::max(sm->max_in, (int)nin); sm->max_hv = std::max(sm->max_hv, (int)std::max(lvd, rvd)); sm->max_rec = std::max(sm->max_rec, (int)(rC + 2 * (size_t)l.d_heads));
+    }
+    if (l.mlp == TGX_MLP_DENSE) {
+      const size_t F = (size_t)l.ff;
+      if ((rc = dev_alloc(c, &w.w_gate, F * W * es)) || (rc = dev_alloc(c, &w.w_up, F * W * es)) || (rc = dev_alloc(c, &w.w_down, W * F * es))) return rc;
+      need(p, {"mlp.gate", "mlp.up", "mlp.down"});
+      sm->max_ff = std::max(sm->max_ff, l.ff);
+    }
+  }
+  return TGX_OK;
+}
+
+// tensors of a parallel-sublayer design by checkpoint name
+int upload_joint(tgx_ctx* c, const char* name, const void* host, const int64_t* shape, int nd, int src_dtype) {
+  StackModel* sm = c->stack;
+  const tgx_stack_desc& d = sm->d;
+  const int64_t W = d.width;
+  const bool probe = nd < 0;
+  auto bad_shape = [&]() { return set_err(c, TGX_ERR_SHAPE, "shape not equal for tensor: %s", name); };
+  auto is = [&](int64_t a, int64_t b) { return b < 0 ? (nd == 1 && shape[0] == a) : (nd == 2 && shape[0] == a && shape[1] == b); };
+  auto done = [&](int rc) { if (!rc) sm->missing.erase(name); return rc; };
+  auto mat = [&](ebyte* dst, int64_t row0, int64_t rows, int64_t cols) {
+    if (probe) return (int)TGX_ERR_SHAPE;
+    if (!is(rows, cols)) return bad_shape();
+    return done(upload_param_ext(c, dst + (size_t)(row0 * cols) * c->esz, host, rows * cols, src_dtype));
+  };
+  auto vec = [&](float* dst, int64_t n, int64_t n2 = -1) {      // an fp32 vector, or (n2 >= 0) an fp32 matrix [n][n2]
+    if (probe) return (int)TGX_ERR_SHAPE;
+    if (!is(n, n2)) return bad_shape();
+    return done(upload_f32(c, dst, host, n2 < 0 ? n : n * n2, src_dtype));
+  };
+  if (!strcmp(name, "embed")) return mat(c->embed, 0, d.vocab, W);
+  if (!strcmp(name, "head")) return mat(sm->head, 0, d.vocab, W);
+  if (!strcmp(name, "final.norm")) return vec(sm->final_norm, W);
+  int li = -1;
+  char rest[128] = {0};
+  if (sscanf(name, "l%d.%127s", &li, rest) != 2 || li < 0 || li >= d.layers) return set_err(c, TGX_ERR_NAME, "Unexpected key: %s", name);
+  StackLayerW& w = sm->L[(size_t)li];
+  tgx_layer_desc& l = w.d;
+  if (!strcmp(rest, "norm1")) return vec(w.norm1, W);
+  if (l.mlp == TGX_MLP_DENSE) {
+    if (!strcmp(rest, "mlp.gate")) return mat(w.w_gate, 0, l.ff, W);
+    if (!strcmp(rest, "mlp.up")) return mat(w.w_up, 0, l.ff, W);
+    if (!strcmp(rest, "mlp.down")) return mat(w.w_down, 0, W, l.ff);
+  }
+  if (l.mixer == TGX_MIXER_ATTENTION) {
+    const int64_t qd = (int64_t)l.heads * l.dim, kd = (int64_t)l.kv_heads * l.dim, kvv = (int64_t)l.kv_heads * l.vdim;
+    if (!strcmp(rest, "mix.q")) return mat(w.w_in, 0, qd, W);
+    if (!strcmp(rest, "mix.o")) return mat(w.w_o, 0, W, (int64_t)l.heads * l.vdim);
+    if (w.kv_src < 0 && !strcmp(rest, "mix.k")) return mat(w.w_in, qd, kd, W);
+    if (w.kv_src < 0 && !strcmp(rest, "mix.v")) return mat(w.w_in, qd + kd, kvv, W);
+  } else if (l.mixer == TGX_MIXER_WKV) {
+    const int64_t HD = (int64_t)l.heads * l.dim;
+    const char* order = "rkvgw";
+    if (!strncmp(rest, "mix.mu.", 7) && rest[7] && !rest[8] && strchr(order, rest[7])) return vec(w.mu + (size_t)(strchr(order, rest[7]) - order) * W, W);
+    if (!strncmp(rest, "mix.", 4) && rest[4] && !rest[5] && strchr("rkvg", rest[4])) return mat(w.w_in, (strchr(order, rest[4]) - order) * HD, HD, W);
+    if (!strcmp(rest, "mix.w1") || !strcmp(rest, "mix.w2")) {      // the inner size of the decay's product is the tensors' own where the description leaves it open
+      if (probe) return TGX_ERR_SHAPE;
+      const bool first = rest[5] == '1';
+      if (nd != 2) return bad_shape();
+      if (l.decay_rank <= 0) {
+        const int64_t R = first ? shape[0] : shape[1];
+        if (R <= 0 || R > 65536) return bad_shape();
+        int rc;
+        if ((rc = dev_alloc(c, &w.w_w1, (size_t)(R * W) * c->esz)) || (rc = dev_alloc(c, &w.w_w2, (size_t)(HD * R) * c->esz))) return rc;
+        l.decay_rank = (int32_t)R;
+        sm->max_lora = std::max(sm->max_lora, l.decay_rank);
+      }
+      return first ? mat(w.w_w1, 0, l.decay_rank, W) : mat(w.w_w2, 0, HD, l.decay_rank);
+    }
+    if (!strcmp(rest, "mix.w0")) return vec(w.w0, HD);
+    if (!strcmp(rest, "mix.u")) return nd == 1 ? vec(w.ubonus, HD) : vec(w.ubonus, l.heads, l.dim);
+    if (!strcmp(rest, "mix.norm")) return vec(w.head_w, HD);
+    if (!strcmp(rest, "mix.o")) return mat(w.w_o, 0, W, HD);
+  } else {
+    const int64_t lq = (int64_t)l.heads * l.dim, lk = (int64_t)l.kv_heads * l.dim, lv = (int64_t)l.kv_heads * l.vdim, lvd = (int64_t)l.heads * l.vdim;
+    const int64_t rGD = (int64_t)l.d_kv_heads * l.d_dim, rvd = (int64_t)l.d_heads * l.d_vdim, r0 = lq + lk + lv, rH = l.d_heads;
+    if (!strcmp(rest, "mix.left.q")) return mat(w.w_in, 0, lq, W);
+    if (!strcmp(rest, "mix.left.k")) return mat(w.w_in, lq, lk, W);
+    if (!strcmp(rest, "mix.left.v")) return mat(w.w_in, lq + lk, lv, W);
+    if (!strcmp(rest, "mix.left.o")) return mat(w.w_o, 0, W, lvd);
+    if (!strcmp(rest, "mix.right.q")) return mat(w.w_in, r0, rGD, W);
+    if (!strcmp(rest, "mix.right.k")) return mat(w.w_in, r0 + rGD, rGD, W);
+    if (!strcmp(rest, "mix.right.v")) return mat(w.w_in, r0 + 2 * rGD, rvd, W);
+    if (!strcmp(rest, "mix.right.b")) return mat(w.w_in, r0 + 2 * rGD + rvd, rH, W);
+    if (!strcmp(rest, "mix.right.a")) return mat(w.w_in, r0 + 2 * rGD + rvd + rH, rH, W);
+    if (!strcmp(rest, "mix.right.g")) return mat(w.w_in, r0 + 2 * rGD + rvd + 2 * rH, rvd, W);
+    if (!strcmp(rest, "mix.right.o")) return mat(w.w_o2, 0, W, rvd);
+    if (!strcmp(rest, "mix.right.q.conv")) return vec(w.conv_w, rGD, l.conv_taps);
+    if (!strcmp(rest, "mix.right.k.conv")) return vec(w.conv_w + (size_t)rGD * l.conv_taps, rGD, l.conv_taps);
+    if (!strcmp(rest, "mix.right.v.conv")) return vec(w.conv_w + (size_t)2 * rGD * l.conv_taps, rvd, l.conv_taps);
+    if (!strcmp(rest, "mix.right.A_log")) return vec(w.a_log, rH);
+    if (!strcmp(rest, "mix.right.dt_bias")) return vec(w.dt_bias, rH);
+    if (!strcmp(rest, "mix.right.norm")) return vec(w.head_w, l.d_vdim);
+  }
+  return set_err(c, TGX_ERR_NAME, "Unexpected key: %s", name);
+}
+
 }  // namespace
 
 // ================================================================================================================================================
@@ -740,17 +1054,46 @@ int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int d
   if (!desc || !layers || !out_ctx) return set_err(nullptr, TGX_ERR_INVALID, "null argument");
   *out_ctx = nullptr;
   const tgx_stack_desc& d = *desc;
-  if (d.family != TGX_FAMILY_ZAKUSUN && d.family != TGX_FAMILY_MODEPEL) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "family %d is not a layered model", d.family);
-  const bool sandwich = d.family == TGX_FAMILY_MODEPEL;
+  if (d.family != TGX_FAMILY_ZAKUSUN && d.family != TGX_FAMILY_MODEPEL && d.family != TGX_FAMILY_VITUDRA) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "family %d is not a layered model", d.family);
+  const bool sandwich = d.family == TGX_FAMILY_MODEPEL, joint = d.family == TGX_FAMILY_VITUDRA;
   if (d.width <= 0 || d.layers <= 0 || d.vocab <= 0 || d.max_seqs <= 0 || d.max_ctx <= 0) return set_err(nullptr, TGX_ERR_INVALID, "non-positive model dimension");
   if (d.compute_dtype != TGX_BF16 && d.compute_dtype != TGX_F16 && d.compute_dtype != TGX_F32) return set_err(nullptr, TGX_ERR_INVALID, "unknown compute dtype %d", d.compute_dtype);
-  if (!sandwich && (d.norm_groups < 1 || d.norm_groups > tgx::NORM_MAX_GROUPS || d.width % d.norm_groups)) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "norm groups %d: 1..%d, dividing the width", d.norm_groups, tgx::NORM_MAX_GROUPS);
-  if (!sandwich && (d.canon_taps < 1 || d.canon_taps > tgx::CONV_MAX_TAPS)) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "convolution taps %d: 1..%d", d.canon_taps, tgx::CONV_MAX_TAPS);
+  if (!sandwich && !joint && (d.norm_groups < 1 || d.norm_groups > tgx::NORM_MAX_GROUPS || d.width % d.norm_groups)) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "norm groups %d: 1..%d, dividing the width", d.norm_groups, tgx::NORM_MAX_GROUPS);
+  if (!sandwich && !joint && (d.canon_taps < 1 || d.canon_taps > tgx::CONV_MAX_TAPS)) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "convolution taps %d: 1..%d", d.canon_taps, tgx::CONV_MAX_TAPS);
   int page = d.page_tokens > 0 ? d.page_tokens : 64;
   if (page & (page - 1)) return set_err(nullptr, TGX_ERR_INVALID, "page_tokens %d is not a power of two", page);
   int first_mix = -1;
   for (int i = 0; i < d.layers; i++) {
     const tgx_layer_desc& l = layers[i];
+    if (joint) {
+      auto attention_ok = [&](const char*& why) {
+        if (l.heads <= 0 || l.dim <= 0 || l.vdim <= 0 || l.kv_heads <= 0 || l.heads % l.kv_heads) { why = "head counts / sizes"; return false; }
+        if (l.dim > 64 * tgx::GQA_MAX_RPL || l.vdim > 64 * tgx::GQA_MAX_RPL) { why = "head size beyond 256"; return false; }
+        if (l.rot_dims < 0 || l.rot_dims > l.dim || (l.rot_dims & 1) || (l.rot_dims > 0 && !(l.rot_base > 0.f))) { why = "rotated dimensions"; return false; }
+        if (l.mask_kind < 0 || l.mask_kind > 2 || (l.mask_kind != 0 && l.mask_size < 1)) { why = "mask"; return false; }
+        if (l.q_temp_coef != 0.f && l.q_temp_every < 1) { why = "query temperature period"; return false; }
+        return true;
+      };
+      const char* why = "";
+      if (l.mixer == TGX_MIXER_ATTENTION) {
+        if (!attention_ok(why)) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: attention: %s", i, why);
+        if (l.kv_share) {
+          const int j = l.kv_share - 1;
+          if (j < 0 || j >= i || layers[j].mixer != TGX_MIXER_ATTENTION || layers[j].kv_share || layers[j].kv_heads != l.kv_heads || layers[j].dim != l.dim || layers[j].vdim != l.vdim)
+            return set_err(nullptr, TGX_ERR_INVALID, "layer %d: reads the keys and values of layer %d, which must be an earlier attention layer with its own projections and the same key / value heads", i, j);
+        }
+      } else if (l.mixer == TGX_MIXER_WKV) {
+        if (l.heads <= 0 || l.dim <= 0 || l.dim > 256 || l.decay_rank < 0) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: wkv: %d heads of %d (1 .. 256), decay rank %d", i, l.heads, l.dim, l.decay_rank);
+      } else if (l.mixer == TGX_MIXER_PARALLEL) {
+        if (!attention_ok(why) || l.kv_share) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: parallel, attention half: %s", i, l.kv_share ? "shared keys are not part of it" : why);
+        if (l.d_heads <= 0 || l.d_kv_heads <= 0 || l.d_heads % l.d_kv_heads || l.d_dim <= 0 || l.d_dim > 256 || l.d_vdim <= 0 || l.conv_taps < 1 || l.conv_taps > tgx::CONV_MAX_TAPS)
+          return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: parallel, delta-rule half: %d heads over %d key heads of %d (1 .. 256) x %d, %d taps (1 .. %d)", i, l.d_heads, l.d_kv_heads, l.d_dim, l.d_vdim, l.conv_taps, tgx::CONV_MAX_TAPS);
+        if ((2LL * l.d_kv_heads * l.d_dim + (long long)l.d_heads * l.d_vdim) * 4 > 60000) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: parallel, delta-rule half: more than 15000 convolved channels", i);
+      } else return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: mixer %d is not part of this family (attention, wkv and parallel are)", i, l.mixer);
+      if (l.mlp != TGX_MLP_NONE && l.mlp != TGX_MLP_DENSE) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: feed-forward kind %d is not implemented", i, l.mlp);
+      if (l.mlp == TGX_MLP_DENSE && l.ff <= 0) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: ff %d", i, l.ff);
+      continue;
+    }
     if (sandwich) {
       if (l.mixer != TGX_MIXER_ATTENTION && l.mixer != TGX_MIXER_MLSTM) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: mixer %d is not part of this family (attention and mlstm are)", i, l.mixer);
       if (l.heads <= 0 || l.dim <= 0 || l.vdim <= 0) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: non-positive mixer size", i);
@@ -799,8 +1142,8 @@ int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int d
   while ((1 << sm->page_shift) < page) sm->page_shift++;
   // what the shared sampler / token rings read from the flat description
   c->d.family = d.family; c->d.hidden = d.width; c->d.layers = d.layers; c->d.vocab = d.vocab; c->d.max_ctx = d.max_ctx; c->d.max_batch = d.max_seqs;
-  c->d.compute_dtype = d.compute_dtype; c->d.tied = sandwich ? 0 : 1; c->d.norm_eps = d.norm_eps;
-  sm->sandwich = sandwich;
+  c->d.compute_dtype = d.compute_dtype; c->d.tied = sandwich || joint ? 0 : 1; c->d.norm_eps = d.norm_eps;
+  sm->sandwich = sandwich; sm->joint = joint;
   c->device = device_ordinal;
   c->dt = d.compute_dtype == TGX_BF16 ? tgx::DT_BF16 : (d.compute_dtype == TGX_F16 ? tgx::DT_F16 : tgx::DT_F32);
   c->esz = d.compute_dtype == TGX_F32 ? 4 : 2;
@@ -816,6 +1159,7 @@ int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int d
   sm->missing.insert("embed"); sm->missing.insert("final.norm");
   sm->L.resize((size_t)d.layers);
   if (sandwich) return create_sandwich_layers(c, layers);
+  if (joint) return create_joint_layers(c, layers);
   for (int i = 0; i < d.layers; i++) {
     StackLayerW& w = sm->L[(size_t)i];
     w.d = layers[i];
@@ -855,6 +1199,7 @@ int stack_upload(tgx_ctx* c, const char* name, const void* host, const int64_t* 
   auto done = [&](int rc) { if (!rc) sm->missing.erase(name); return rc; };
   if (src_dtype != TGX_BF16 && src_dtype != TGX_F32 && src_dtype != TGX_F16) return set_err(c, TGX_ERR_INVALID, "unknown source dtype %d", src_dtype);
   if (sm->sandwich) return upload_sandwich(c, name, host, shape, nd, src_dtype);
+  if (sm->joint) return upload_joint(c, name, host, shape, nd, src_dtype);
   if (!strcmp(name, "embed")) { if (probe) return TGX_ERR_SHAPE; if (!is(d.vocab, W)) return bad_shape(); return done(upload_param_ext(c, c->embed, host, d.vocab * W, src_dtype)); }
   if (!strcmp(name, "final.norm")) { if (probe) return TGX_ERR_SHAPE; if (!is(W, -1)) return bad_shape(); return done(upload_f32(c, sm->final_norm, host, W, src_dtype)); }
   int li = -1;
@@ -918,7 +1263,7 @@ int stack_finalize(tgx_ctx* c) {
   const size_t W = (size_t)d.width, B = (size_t)d.max_seqs, V = (size_t)d.vocab;
   int rc;
   // angles of the position vector: pos * base^(-2i / width), the factor rounded to fp32 once
-  if (!sm->sandwich) {
+  if (!sm->sandwich && !sm->joint) {
     std::vector<float> fq(W / 2 + 1);
     for (size_t i = 0; i < fq.size(); i++) fq[i] = (float)pow(10000.0, -2.0 * (double)i / (double)W);
     if ((rc = dev_alloc(c, &sm->freq, fq.size()))) return rc;
@@ -934,18 +1279,56 @@ int stack_finalize(tgx_ctx* c) {
   memset(sm->tbl_host, 0, B * (size_t)sm->tbl_stride * 4);
   sm->row_pages.assign(B, 0); sm->row_par.assign(B, 0); sm->row_dirty.assign(B, 0);
   for (int p = sm->n_pages - 1; p >= 0; p--) sm->free_pages.push_back(p);
-  const size_t nb = sm->sandwich ? 0 : (size_t)d.canon_taps - 1;
+  const size_t nb = sm->sandwich || sm->joint ? 0 : (size_t)d.canon_taps - 1;
   for (auto& r : sm->rot) {      // angle of (position, pair i) = position * base^(-2i / dims), evaluated in double, stored as fp32 cosine and sine
     const size_t half = (size_t)r.dims / 2;
     std::vector<float> cs((size_t)d.max_ctx * half * 2);
     for (size_t i = 0; i < half; i++) {
-      const double f = pow((double)r.base, -2.0 * (double)i / (double)r.dims);
+      const double f = pow((double)r.base, -2.0 * (double)i / (double)r.dims) / (double)r.factor;
       for (size_t p = 0; p < (size_t)d.max_ctx; p++) { cs[(p * half + i) * 2] = (float)cos((double)p * f); cs[(p * half + i) * 2 + 1] = (float)sin((double)p * f); }
     }
     if ((rc = dev_alloc(c, &r.cs, cs.size()))) return rc;
     HIP_OK(c, hipMemcpy(r.cs, cs.data(), cs.size() * 4, hipMemcpyHostToDevice));
   }
   for (auto& w : sm->L) {
+    if (sm->joint) {
+      const tgx_layer_desc& l = w.d;
+      if (l.mixer != TGX_MIXER_WKV && w.kv_src < 0) {      // keys and values of an attention layer / a parallel mixer's attention half (a sharing layer borrows below)
+        const size_t ke = (size_t)sm->n_pages * sm->page * (size_t)l.kv_heads * l.dim * c->esz, ve = (size_t)sm->n_pages * sm->page * (size_t)l.kv_heads * l.vdim * c->esz;
+        if ((rc = dev_alloc(c, &w.pool, ke)) || (rc = dev_alloc(c, &w.poolV, ve))) return rc;
+        HIP_OK(c, hipMemset(w.pool, 0, ke));
+        HIP_OK(c, hipMemset(w.poolV, 0, ve));
+        // every layer that reads this pool must be able to take the matrix-core kernel's query rows (their strides differ)
+        bool mfma = true;
+        for (auto& r : sm->L) {
+          if (&r != &w && !(r.kv_src >= 0 && &sm->L[(size_t)r.kv_src] == &w)) continue;
+          const tgx_layer_desc& q = r.d;
+          long long ldq = (long long)q.heads * q.dim + (r.kv_src >= 0 ? 0 : (long long)q.kv_heads * (q.dim + q.vdim));
+          if (q.mixer == TGX_MIXER_PARALLEL) ldq += 2LL * q.d_kv_heads * q.d_dim + 2LL * q.d_heads * q.d_vdim + 2LL * q.d_heads;
+          mfma = mfma && gqa_mfma_shapes_ok(c->dt, q.dim, q.vdim, sm->page_shift, ldq);
+        }
+        if (mfma) {
+          if ((rc = dev_alloc(c, &w.poolVT, ve))) return rc;
+          HIP_OK(c, hipMemset(w.poolVT, 0, ve));
+        }
+      }
+      if (l.mixer == TGX_MIXER_WKV) {
+        const size_t se = B * (size_t)l.heads * l.dim * l.dim;
+        if ((rc = dev_alloc(c, &w.mS, se)) || (rc = dev_alloc(c, &w.shift, 2 * B * W))) return rc;
+        HIP_OK(c, hipMemset(w.mS, 0, se * 4));
+        HIP_OK(c, hipMemset(w.shift, 0, 2 * B * W * 4));
+        if (l.decay_rank <= 0) return set_err(c, TGX_ERR_STATE, "a wkv layer's decay product has no inner size");
+      } else if (l.mixer == TGX_MIXER_PARALLEL) {
+        const size_t se = B * (size_t)l.d_heads * l.d_dim * l.d_vdim, rC = 2 * (size_t)l.d_kv_heads * l.d_dim + (size_t)l.d_heads * l.d_vdim, ce = 2 * B * (size_t)(l.conv_taps - 1) * rC;
+        if ((rc = dev_alloc(c, &w.mS, se))) return rc;
+        HIP_OK(c, hipMemset(w.mS, 0, se * 4));
+        if (ce > 0) {
+          if ((rc = dev_alloc(c, &w.conv_state, ce))) return rc;
+          HIP_OK(c, hipMemset(w.conv_state, 0, ce * 4));
+        }
+      }
+      continue;
+    }
     if (sm->sandwich) {
       if (w.d.mixer == TGX_MIXER_ATTENTION) {      // keys and values of the layer, one page table for both
         const size_t ke = (size_t)sm->n_pages * sm->page * (size_t)w.d.kv_heads * w.d.dim * c->esz, ve = (size_t)sm->n_pages * sm->page * (size_t)w.d.kv_heads * w.d.vdim * c->esz;
@@ -979,6 +1362,8 @@ int stack_finalize(tgx_ctx* c) {
       HIP_OK(c, hipMemset(w.conv_state, 0, se * 4));
     }
   }
+  for (auto& w : sm->L)      // layers that read another layer's keys and values borrow its pools
+    if (w.kv_src >= 0) { const StackLayerW& o = sm->L[(size_t)w.kv_src]; w.pool = o.pool; w.poolV = o.poolV; w.poolVT = o.poolVT; }
   if ((rc = dev_alloc(c, &sm->moe_off, (size_t)sm->max_E + 2)) || (rc = dev_alloc(c, &sm->n_tiles, 1))) return rc;
   HIP_OK(c, hipEventCreateWithFlags(&sm->meta_ev, hipEventDisableTiming));
   // the rows of the shared sampler (logits, argmax partials, current token) and the token rings
@@ -1017,11 +1402,14 @@ void stack_destroy(tgx_ctx* c) {
   if (!sm) return;
   auto fr = [](void* p) { if (p) (void)hipFree(p); };
   for (auto& w : sm->L) {
+    if (w.kv_src >= 0) w.pool = w.poolV = w.poolVT = nullptr;      // borrowed
+    fr(w.w_o2); fr(w.w_w1); fr(w.w_w2); fr(w.mu); fr(w.w0); fr(w.ubonus); fr(w.conv_w); fr(w.a_log); fr(w.dt_bias); fr(w.shift);
     fr(w.norm1); fr(w.norm2); fr(w.canon1); fr(w.canon2); fr(w.dwa); fr(w.w_in); fr(w.w_ukT); fr(w.w_uv); fr(w.w_o); fr(w.lat_norm); fr(w.sink);
     fr(w.w_gate); fr(w.w_up); fr(w.w_down); fr(w.w_router); fr(w.b_router); fr(w.pool); fr(w.poolT); fr(w.conv_state);
     fr(w.b_in); fr(w.poolV); fr(w.poolVT); fr(w.vmix); fr(w.head_w); fr(w.mS); fr(w.mn); fr(w.mm); fr(w.act); fr(w.ws_gate); fr(w.ws_up); fr(w.ws_down);
   }
   for (auto& r : sm->rot) fr(r.cs);
+  fr(sm->mixed); fr(sm->lora); fr(sm->rec_in);
   fr(sm->head); fr(sm->norm_g); fr(sm->a2); fr(sm->ytmp); fr(sm->ysh); fr(sm->sgw); fr(sm->vfirst); fr(sm->hs);
   fr(sm->final_norm); fr(sm->freq); fr(sm->tbl_dev); fr(sm->meta_dev); fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw);
   fr(sm->yh); fr(sm->yd); fr(sm->xn); fr(sm->lg); fr(sm->part); fr(sm->zr); fr(sm->sel); fr(sm->moe_off); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->n_tiles);
@@ -1181,8 +1569,8 @@ int stack_read_latent(tgx_ctx* c, int row, int layer, float* out) {
   if (row < 0 || row >= sm->d.max_seqs || layer < 0 || layer >= sm->d.layers || !out) return set_err(c, TGX_ERR_INVALID, "read_kv: row / layer out of range");
   HIP_OK(c, hipStreamSynchronize(c->stream));
   const StackLayerW& w = sm->L[(size_t)layer];
-  if (sm->sandwich && w.d.mixer != TGX_MIXER_ATTENTION) return set_err(c, TGX_ERR_UNSUPPORTED, "read_kv: layer %d caches no rows (its state is recurrent)", layer);
-  const size_t R = sm->sandwich ? (size_t)w.d.kv_heads * w.d.dim : (size_t)w.d.kv_rank;      // an attention layer's cached keys, all key heads of a token in a row
+  if ((sm->sandwich && w.d.mixer != TGX_MIXER_ATTENTION) || (sm->joint && !w.pool)) return set_err(c, TGX_ERR_UNSUPPORTED, "read_kv: layer %d caches no rows (its state is recurrent)", layer);
+  const size_t R = sm->sandwich || sm->joint ? (size_t)w.d.kv_heads * w.d.dim : (size_t)w.d.kv_rank;      // an attention layer's cached keys, all key heads of a token in a row
   std::vector<unsigned char> buf(R * c->esz);
   for (int64_t t = 0; t < c->row_past[(size_t)row]; t++) {
     const size_t page = (size_t)sm->tbl_host[(size_t)row * sm->tbl_stride + (size_t)(t >> sm->page_shift)];
@@ -1198,10 +1586,21 @@ int64_t stack_bytes_per_token(const tgx_ctx* c, int64_t T) {
   const StackModel* sm = c->stack;
   const int64_t W = sm->d.width, es = (int64_t)c->esz;
   int64_t b = (int64_t)sm->d.vocab * W * es;
-  if (sm->sandwich) b *= 2;      // embedding row aside, the head is a matrix of its own
+  if (sm->sandwich || sm->joint) b *= 2;      // embedding row aside, the head is a matrix of its own
   for (const auto& w : sm->L) {
     const tgx_layer_desc& l = w.d;
     const int64_t H = l.heads, qd = H * l.dim, R = l.kv_rank, vd = H * l.vdim;
+    if (sm->joint) {      // an attention layer reads at most its mask's span of keys; a recurrent state is read and written
+      const int64_t keys = l.mask_kind ? std::min<int64_t>(T, l.mask_size) : T, kvw = (int64_t)l.kv_heads * (l.dim + l.vdim);
+      if (l.mixer == TGX_MIXER_ATTENTION) b += ((qd + (w.kv_src >= 0 ? 0 : kvw)) * W + W * vd) * es + keys * kvw * es;
+      else if (l.mixer == TGX_MIXER_WKV) b += (5 * qd * W + (int64_t)l.decay_rank * (W + qd)) * es + 2 * qd * l.dim * 4;
+      else {
+        const int64_t rvd = (int64_t)l.d_heads * l.d_vdim, rgd = (int64_t)l.d_kv_heads * l.d_dim;
+        b += ((qd + kvw + 2 * rgd + 2 * rvd + 2 * l.d_heads) * W + W * (vd + rvd)) * es + keys * kvw * es + 2 * rvd * l.d_dim * 4;
+      }
+      if (l.mlp == TGX_MLP_DENSE) b += 3 * (int64_t)l.ff * W * es;
+      continue;
+    }
     if (sm->sandwich) {
       if (l.mixer == TGX_MIXER_ATTENTION) b += ((qd + (int64_t)l.kv_heads * (l.dim + l.vdim) + vd) * W + W * vd) * es + T * l.kv_heads * (l.dim + l.vdim) * es;
       else b += ((2 * qd + 2 * vd + 2 * H) * W + W * vd) * es + 2 * H * (int64_t)l.dim * l.vdim * 4;      // the state is read and written

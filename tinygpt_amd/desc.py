@@ -270,11 +270,13 @@ def known_desc(key: str, compute_dtype: str | None = None, max_batch: int = 1) -
 # ---- layered models (include/tgx.h tgx_stack_desc / tgx_layer_desc) -------------------------------------------------------------
 FAMILY_ZAKUSUN = 6
 FAMILY_MODEPEL = 7
-STACK_FAMILY = {"zakusun": FAMILY_ZAKUSUN, "modepel": FAMILY_MODEPEL}
-MIXER_BY_NAME = {"latent_attention": 1, "attention": 2, "mlstm": 3}
+FAMILY_VITUDRA = 8
+STACK_FAMILY = {"zakusun": FAMILY_ZAKUSUN, "modepel": FAMILY_MODEPEL, "vitudra": FAMILY_VITUDRA}
+MIXER_BY_NAME = {"latent_attention": 1, "attention": 2, "mlstm": 3, "wkv": 4, "parallel": 5}
 MLP_BY_NAME = {None: 0, "moe": 1, "dense": 2}
+MASK_BY_NAME = {None: 0, "window": 1, "chunk": 2}
 # which mixers a design is made of (config.json "architecture" -> layer "type")
-MIXERS_OF = {"zakusun": ("latent_attention",), "modepel": ("attention", "mlstm")}
+MIXERS_OF = {"zakusun": ("latent_attention",), "modepel": ("attention", "mlstm"), "vitudra": ("attention", "wkv", "parallel")}
 
 
 class CLayerDesc(ctypes.Structure):
@@ -284,7 +286,12 @@ class CLayerDesc(ctypes.Structure):
                 ("top", ctypes.c_int32), ("ff", ctypes.c_int32), ("limit", ctypes.c_float),
                 ("kv_heads", ctypes.c_int32), ("rot_dims", ctypes.c_int32), ("rot_base", ctypes.c_float), ("v_mix", ctypes.c_int32),
                 ("gate_cap", ctypes.c_float), ("identity", ctypes.c_int32), ("groups", ctypes.c_int32), ("groups_keep", ctypes.c_int32),
-                ("router_scale", ctypes.c_float), ("shared_ff", ctypes.c_int32)]
+                ("router_scale", ctypes.c_float), ("shared_ff", ctypes.c_int32),
+                ("mask_kind", ctypes.c_int32), ("mask_size", ctypes.c_int32), ("softcap", ctypes.c_float), ("dist_bias", ctypes.c_int32),
+                ("q_temp_coef", ctypes.c_float), ("q_temp_every", ctypes.c_int32), ("rot_pairs", ctypes.c_int32), ("rot_factor", ctypes.c_float),
+                ("kv_share", ctypes.c_int32), ("decay_rank", ctypes.c_int32), ("d_heads", ctypes.c_int32), ("d_kv_heads", ctypes.c_int32),
+                ("d_dim", ctypes.c_int32), ("d_vdim", ctypes.c_int32), ("conv_taps", ctypes.c_int32), ("left_scale", ctypes.c_float),
+                ("right_scale", ctypes.c_float)]
 
 
 class CStackDesc(ctypes.Structure):
@@ -292,7 +299,7 @@ class CStackDesc(ctypes.Structure):
     _fields_ = [("family", ctypes.c_int32), ("width", ctypes.c_int32), ("layers", ctypes.c_int32), ("vocab", ctypes.c_int32),
                 ("compute_dtype", ctypes.c_int32), ("max_seqs", ctypes.c_int32), ("max_ctx", ctypes.c_int32),
                 ("budget_tokens", ctypes.c_int32), ("page_tokens", ctypes.c_int32), ("norm_groups", ctypes.c_int32),
-                ("norm_eps", ctypes.c_float), ("canon_taps", ctypes.c_int32), ("logit_scale", ctypes.c_float)]
+                ("norm_eps", ctypes.c_float), ("canon_taps", ctypes.c_int32), ("logit_scale", ctypes.c_float), ("residual_mult", ctypes.c_float)]
 
 
 @dataclass
@@ -321,12 +328,35 @@ class LayerDesc:
     groups_keep: int = 1
     router_scale: float = 1.0
     shared_ff: int = 0
+    # attention of the parallel-sublayer design (Vitudra): mask, score shaping, rotary variant, shared keys and values
+    mask: "str | None" = None     # None: causal; "window": the last mask_size positions; "chunk": the position's own block of mask_size
+    mask_size: int = 0
+    softcap: float = 0.0
+    dist_bias: bool = False
+    q_temp_coef: float = 0.0
+    q_temp_every: int = 0
+    rot_pairs: bool = False       # neighbours (2i, 2i + 1) turn together instead of (i, i + rot_dims / 2)
+    rot_factor: float = 1.0       # every angle is divided by this
+    kv_from: "int | None" = None  # the layer whose keys and values this one reads
+    # token-shift mixer ("wkv")
+    decay_rank: int = 0
+    # the gated-delta-rule half of a "parallel" mixer (heads .. rot_* above describe its attention half)
+    d_heads: int = 0
+    d_kv_heads: int = 0
+    d_dim: int = 0
+    d_vdim: int = 0
+    conv_taps: int = 0
+    left_scale: float = 1.0
+    right_scale: float = 1.0
 
     def to_c(self) -> CLayerDesc:
         return CLayerDesc(MIXER_BY_NAME[self.mixer], self.heads, self.dim, self.vdim, self.kv_rank, self.scale,
                           MLP_BY_NAME[self.mlp], self.experts, self.top, self.ff, self.limit,
                           self.kv_heads, self.rot_dims, self.rot_base, int(self.v_mix), self.gate_cap, self.identity, self.groups,
-                          self.groups_keep, self.router_scale, self.shared_ff)
+                          self.groups_keep, self.router_scale, self.shared_ff,
+                          MASK_BY_NAME[self.mask], self.mask_size, self.softcap, int(self.dist_bias), self.q_temp_coef, self.q_temp_every,
+                          int(self.rot_pairs), self.rot_factor, 0 if self.kv_from is None else self.kv_from + 1, self.decay_rank,
+                          self.d_heads, self.d_kv_heads, self.d_dim, self.d_vdim, self.conv_taps, self.left_scale, self.right_scale)
 
 
 @dataclass
@@ -345,6 +375,7 @@ class StackDesc:
     norm_eps: float = 1e-6
     canon_taps: int = 1
     logit_scale: float = 1.0
+    residual_mult: float = 1.0   # Vitudra: the factor on what a layer adds to the stream
     name: str = ""
 
     # the fields the flat description shares (bench / reporting code reads them)
@@ -358,7 +389,7 @@ class StackDesc:
         arr = (CLayerDesc * len(self.layers))(*[l.to_c() for l in self.layers])
         sd = CStackDesc(STACK_FAMILY[self.family], self.width, len(self.layers), self.vocab, DTYPE_BY_NAME[self.compute_dtype], self.max_seqs,
                         self.max_ctx, self.budget_tokens, self.page_tokens, self.norm_groups, self.norm_eps, self.canon_taps,
-                        self.logit_scale)
+                        self.logit_scale, self.residual_mult)
         return sd, arr
 
     def tensor_shapes(self) -> "dict[str, tuple]":
@@ -367,6 +398,8 @@ class StackDesc:
         out["embed"] = (self.vocab, W)
         if self.family == "modepel":
             return self._modepel_shapes(out)
+        if self.family == "vitudra":
+            return _vitudra_shapes(self, out)
         for i, l in enumerate(self.layers):
             p = f"l{i}."
             out[p + "norm1"] = (W,)
@@ -419,6 +452,81 @@ class StackDesc:
         return out
 
 
+def _vitudra_shapes(self: StackDesc, out: dict) -> dict:
+    """checkpoint names and shapes of a Vitudra model, in file order"""
+    W = self.width
+    for i, l in enumerate(self.layers):
+        p = f"l{i}."
+        out[p + "norm1"] = (W,)
+        if l.mixer == "attention":
+            out[p + "mix.q"] = (l.heads * l.dim, W)
+            if l.kv_from is None:
+                out[p + "mix.k"] = (l.kv_heads * l.dim, W); out[p + "mix.v"] = (l.kv_heads * l.vdim, W)
+            out[p + "mix.o"] = (W, l.heads * l.vdim)
+        elif l.mixer == "wkv":
+            HD = l.heads * l.dim
+            for s in "rkvgw":
+                out[p + "mix.mu." + s] = (W,)
+            for s in "rkvg":
+                out[p + "mix." + s] = (HD, W)
+            out[p + "mix.w1"] = (l.decay_rank, W); out[p + "mix.w2"] = (HD, l.decay_rank); out[p + "mix.w0"] = (HD,)
+            out[p + "mix.u"] = (l.heads, l.dim); out[p + "mix.norm"] = (HD,); out[p + "mix.o"] = (W, HD)
+        else:
+            q = p + "mix.left."
+            out[q + "q"] = (l.heads * l.dim, W); out[q + "k"] = (l.kv_heads * l.dim, W); out[q + "v"] = (l.kv_heads * l.vdim, W); out[q + "o"] = (W, l.heads * l.vdim)
+            q = p + "mix.right."
+            gd, vd = l.d_kv_heads * l.d_dim, l.d_heads * l.d_vdim
+            for s, n in (("q", gd), ("k", gd), ("v", vd)):
+                out[q + s] = (n, W); out[q + s + ".conv"] = (n, l.conv_taps)
+            out[q + "b"] = (l.d_heads, W); out[q + "a"] = (l.d_heads, W); out[q + "A_log"] = (l.d_heads,); out[q + "dt_bias"] = (l.d_heads,)
+            out[q + "norm"] = (l.d_vdim,); out[q + "g"] = (vd, W); out[q + "o"] = (W, vd)
+        if l.mlp == "dense":
+            out[p + "mlp.gate"] = (l.ff, W); out[p + "mlp.up"] = (l.ff, W); out[p + "mlp.down"] = (W, l.ff)
+    out["final.norm"] = (W,)
+    out["head"] = (self.vocab, W)
+    return out
+
+
+
+def _attention_fields(ld: LayerDesc, m: dict, mask: str):
+    """the attention entries of a Vitudra mixer (an "attention" layer's, or the "left" half of a "parallel" one); what is absent is off"""
+    ld.heads = int(m["heads"]); ld.kv_heads = int(m.get("kv_heads", m["heads"])); ld.dim = int(m["dim"]); ld.vdim = int(m.get("vdim", m["dim"]))
+    ld.scale = float(m["scale"]); ld.softcap = float(m.get("softcap") or 0.0)
+    if m.get("mask"):
+        ld.mask = mask; ld.mask_size = int(m["mask"]["size"])
+    rot = m.get("rot")
+    if rot:
+        ld.rot_dims = int(rot["dims"]); ld.rot_base = float(rot["base"]); ld.rot_pairs = True
+        ld.rot_factor = float((rot.get("scaling") or {}).get("factor", 1.0))
+    qt = m.get("q_temp")
+    if qt:
+        ld.q_temp_coef = float(qt["coef"]); ld.q_temp_every = int(qt["every"])
+
+
+def _vitudra_layer(i: int, l: dict, decay_rank: int = 0) -> LayerDesc:
+    """one entry of a Vitudra config's "layers": {"type": "attention" | "wkv" | "parallel", "mixer": {...}, "mlp": null | {"kind": "dense", "ff"}}.
+    An attention layer has a sliding window, a distance bias and a query temperature and may read another layer's keys and values ("kv_from");
+    a parallel mixer's attention half ("left") has neighbour-pair rotation with linear scaling, a soft cap and a chunked mask."""
+    m, f = l["mixer"], l.get("mlp")
+    ld = LayerDesc(mixer=l["type"])
+    if l["type"] == "attention":
+        _attention_fields(ld, m, "window")
+        ld.dist_bias = True
+        ld.kv_from = int(m["kv_from"]) if m.get("kv_from") is not None else None
+    elif l["type"] == "wkv":
+        ld.heads = int(m["heads"]); ld.dim = int(m["dim"]); ld.vdim = ld.dim; ld.kv_heads = ld.heads; ld.decay_rank = int(decay_rank)
+    else:
+        _attention_fields(ld, m["left"], "chunk")
+        r = m["right"]
+        ld.d_heads = int(r["heads"]); ld.d_kv_heads = int(r.get("kv_heads", r["heads"])); ld.d_dim = int(r["dim"]); ld.d_vdim = int(r.get("vdim", r["dim"]))
+        ld.conv_taps = int(r.get("conv", 1)); ld.left_scale = float(m.get("left_scale", 1.0)); ld.right_scale = float(m.get("right_scale", 1.0))
+    if f is not None:
+        if f.get("kind") != "dense":
+            raise ValueError(f"layer {i}: feed-forward kind {f.get('kind')!r} is not implemented")
+        ld.mlp = "dense"; ld.ff = int(f["ff"])
+    return ld
+
+
 def _modepel_layer(i: int, l: dict) -> LayerDesc:
     """one entry of a Modepel config's "layers": {"type": "attention" | "mlstm", "mixer": {...}, "mlp": null | {"kind": "dense" | "moe", ...}}"""
     m, f = l["mixer"], l.get("mlp")
@@ -444,14 +552,22 @@ def _modepel_layer(i: int, l: dict) -> LayerDesc:
     return ld
 
 
-def stack_desc_from_config(cfg: dict, compute_dtype: str = "bf16", max_seqs: int = 4, max_ctx: int = 4096, budget_tokens: int = 0) -> StackDesc:
-    """config.json of a layered model ("architecture": "Zakusun" | "Modepel") -> StackDesc.  Every size and constant comes from the file."""
+def stack_desc_from_config(cfg: dict, compute_dtype: str = "bf16", max_seqs: int = 4, max_ctx: int = 4096, budget_tokens: int = 0, tensor_shapes=None) -> StackDesc:
+    """config.json of a layered model ("architecture": "Zakusun" | "Modepel" | "Vitudra") -> StackDesc.  Every size and constant comes from the file;
+    tensor_shapes (checkpoint name -> shape, optional) gives the sizes that only a tensor's shape tells (a wkv layer's decay rank; left open without it:
+    the device library then takes it from the tensor at upload)."""
     arch = str(cfg.get("architecture")).lower()
     if arch not in MIXERS_OF:
         raise ValueError(f"Unsupported architecture: {cfg.get('architecture')!r}")
     for i, l in enumerate(cfg["layers"]):
         if l["type"] not in MIXERS_OF[arch]:
             raise ValueError(f"layer {i}: mixer {l['type']!r} is not implemented")
+    if arch == "vitudra":
+        ts = tensor_shapes or {}
+        layers = [_vitudra_layer(i, l, (ts.get(f"l{i}.mix.w1") or (0,))[0]) for i, l in enumerate(cfg["layers"])]
+        return StackDesc(family="vitudra", width=int(cfg["width"]), vocab=int(cfg["vocab"]), layers=layers, compute_dtype=compute_dtype, max_seqs=max_seqs,
+                         max_ctx=max_ctx, budget_tokens=budget_tokens, norm_groups=1, norm_eps=float(cfg["norm"]["eps"]), canon_taps=1, logit_scale=1.0,
+                         residual_mult=float(cfg.get("residual_mult", 1.0)), name="vitudra")
     if arch == "modepel":
         return StackDesc(family="modepel", width=int(cfg["width"]), vocab=int(cfg["vocab"]), layers=[_modepel_layer(i, l) for i, l in enumerate(cfg["layers"])],
                          compute_dtype=compute_dtype, max_seqs=max_seqs, max_ctx=max_ctx, budget_tokens=budget_tokens, norm_groups=1,
