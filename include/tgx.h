@@ -137,6 +137,7 @@ typedef struct tgx_model_desc {
  *   dense gated feed-forward  down(silu(gate h) * (up h)) */
 typedef enum tgx_mixer { TGX_MIXER_LATENT_ATTENTION = 1, TGX_MIXER_ATTENTION = 2, TGX_MIXER_MLSTM = 3, TGX_MIXER_WKV = 4, TGX_MIXER_PARALLEL = 5 } tgx_mixer;
 typedef enum tgx_mlp { TGX_MLP_NONE = 0, TGX_MLP_MOE = 1, TGX_MLP_DENSE = 2 } tgx_mlp;
+typedef enum tgx_mask { TGX_MASK_CAUSAL = 0, TGX_MASK_WINDOW = 1, TGX_MASK_CHUNK = 2 } tgx_mask;
 
 typedef struct tgx_layer_desc {
   int32_t mixer;     /* tgx_mixer                                                                 */
@@ -162,7 +163,7 @@ typedef struct tgx_layer_desc {
   float router_scale;  /* experts: weights = scores * router_scale                                */
   int32_t shared_ff; /* experts: width of the shared expert (0: none)                             */
   /* ABI 6 (zero for the kinds that do not read them) */
-  int32_t mask_kind; /* attention: 0 causal, 1 sliding window, 2 chunks                           */
+  int32_t mask_kind; /* attention: tgx_mask                                                       */
   int32_t mask_size; /* attention: window / chunk length in positions                             */
   float softcap;     /* attention: soft cap of the scaled score (<= 0: none)                      */
   int32_t dist_bias; /* attention: 1 = minus 2^(-8 (h + 1) / heads) * (i - j)                     */

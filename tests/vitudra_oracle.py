@@ -46,12 +46,6 @@ def causal_mask(T):
     return np.tril(np.ones((T, T), bool))
 
 
-def mask_of(m, T):
-    if not m:
-        return causal_mask(T)
-    return window_mask(T, int(m["size"])) if m.get("kind", "window") == "window" else chunk_mask(T, int(m["size"]))
-
-
 def rotate_pairs(x, dims, base, factor):
     """x [T][heads][D]: neighbours (2i, 2i + 1) of the first `dims` channels turn by position * base^(-2i / dims) / factor"""
     T = x.shape[0]
@@ -106,7 +100,8 @@ def attention_mixer(h, m, t, pre, eps, kv=None):
     qt = m.get("q_temp")
     if qt:
         q = q * query_temperature(T, qt["coef"], qt["every"])[:, None, None]
-    o = softmax_attention(q, kv[0], kv[1], mask_of(dict(m.get("mask") or {}, kind="window") if m.get("mask") else None, T), m["scale"], 0.0, distance_slopes(H))
+    vis = window_mask(T, m["mask"]["size"]) if m.get("mask") else causal_mask(T)
+    o = softmax_attention(q, kv[0], kv[1], vis, m["scale"], 0.0, distance_slopes(H))
     return o.reshape(T, H * E) @ t[pre + "o"].T, kv
 
 
@@ -122,7 +117,7 @@ def rotary_chunk_attention(h, m, t, pre):
         factor = (rot.get("scaling") or {}).get("factor", 1.0)
         q = rotate_pairs(q, rot["dims"], rot["base"], factor)
         k = rotate_pairs(k, rot["dims"], rot["base"], factor)
-    vis = mask_of(dict(m["mask"], kind="chunk") if m.get("mask") else None, T)
+    vis = chunk_mask(T, m["mask"]["size"]) if m.get("mask") else causal_mask(T)
     o = softmax_attention(q, k, v, vis, m["scale"], m.get("softcap", 0.0))
     return o.reshape(T, H * E) @ t[pre + "o"].T
 
@@ -213,3 +208,84 @@ def forward(cfg, t, ids, layers_out=None):
         if layers_out is not None:
             layers_out.append(x.copy())
     return offset_norm(x, t["final.norm"], eps) @ t["head"].T
+
+
+# ---- random models -----------------------------------------------------------------------------------------------------------------
+def tensor_shapes(cfg, decay_rank=5):
+    """checkpoint name -> shape; the decay rank of the wkv layers is not part of the configuration (the tensors carry it)"""
+    W, out = cfg["width"], {"embed": (cfg["vocab"], cfg["width"])}
+    for i, L in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", L["mixer"]
+        out[p + "norm1"] = (W,)
+        if L["type"] == "attention":
+            H, G, D, E = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            out[p + "mix.q"] = (H * D, W)
+            if "kv_from" not in m:
+                out[p + "mix.k"] = (G * D, W); out[p + "mix.v"] = (G * E, W)
+            out[p + "mix.o"] = (W, H * E)
+        elif L["type"] == "wkv":
+            HD = m["heads"] * m["dim"]
+            for s in "rkvgw":
+                out[p + "mix.mu." + s] = (W,)
+            for s in "rkvg":
+                out[p + "mix." + s] = (HD, W)
+            out.update({p + "mix.w1": (decay_rank, W), p + "mix.w2": (HD, decay_rank), p + "mix.w0": (HD,), p + "mix.u": (m["heads"], m["dim"]),
+                        p + "mix.norm": (HD,), p + "mix.o": (W, HD)})
+        else:
+            l, r = m["left"], m["right"]
+            out.update({p + "mix.left.q": (l["heads"] * l["dim"], W), p + "mix.left.k": (l["kv_heads"] * l["dim"], W), p + "mix.left.v": (l["kv_heads"] * l["vdim"], W),
+                        p + "mix.left.o": (W, l["heads"] * l["vdim"])})
+            gd, vd, q = r["kv_heads"] * r["dim"], r["heads"] * r["vdim"], p + "mix.right."
+            for s, n in (("q", gd), ("k", gd), ("v", vd)):
+                out[q + s] = (n, W); out[q + s + ".conv"] = (n, r["conv"])
+            out.update({q + "b": (r["heads"], W), q + "a": (r["heads"], W), q + "A_log": (r["heads"],), q + "dt_bias": (r["heads"],), q + "norm": (r["vdim"],),
+                        q + "g": (vd, W), q + "o": (W, vd)})
+        if L.get("mlp"):
+            F = L["mlp"]["ff"]
+            out.update({p + "mlp.gate": (F, W), p + "mlp.up": (F, W), p + "mlp.down": (W, F)})
+    out["final.norm"] = (W,)
+    out["head"] = (cfg["vocab"], W)
+    return out
+
+
+def bf16_round(a):
+    """round-to-nearest-even onto the bfloat16 grid, so that every storage dtype of the library holds the same numbers"""
+    u = np.asarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    u = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    return u.astype(np.uint32).view(np.float32).reshape(np.shape(a))
+
+
+def random_tensors(cfg, seed=0, overrides=None, decay_rank=5):
+    """weights on the bfloat16 grid, scaled so that every mechanism matters: projections ~ 1 / sqrt(inputs), norm weights around zero, decays spread over (0, 1)"""
+    rng = np.random.default_rng(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg, decay_rank).items():
+        leaf = name.split(".")[-1]
+        if name == "embed":
+            v = rng.standard_normal(shape)
+        elif leaf == "conv":
+            v = rng.standard_normal(shape) * 0.6
+        elif leaf == "u":
+            v = rng.standard_normal(shape) * 0.5
+        elif leaf == "w2":
+            v = rng.standard_normal(shape) * 0.7
+        elif len(shape) == 2:
+            v = rng.standard_normal(shape) / np.sqrt(shape[1])
+        elif leaf == "norm1" or name == "final.norm":
+            v = rng.uniform(-0.3, 0.3, shape)
+        elif ".mu." in name:
+            v = rng.uniform(0.0, 1.0, shape)
+        elif leaf == "w0":
+            v = rng.uniform(-3.0, 0.3, shape)
+        elif leaf == "A_log":
+            v = rng.uniform(-2.5, 0.3, shape)
+        elif leaf == "dt_bias":
+            v = rng.uniform(-1.0, 1.0, shape)
+        elif leaf == "norm":
+            v = rng.uniform(0.5, 1.5, shape)
+        else:
+            v = rng.standard_normal(shape) * 0.3
+        out[name] = bf16_round(v)
+    for k, v in (overrides or {}).items():
+        out[k] = bf16_round(v)
+    return out

@@ -21,7 +21,7 @@ struct StepMeta {          // device arrays of one step (T tokens, S entries)
 };
 
 // attention masks of the layered designs: the first key the query at position `pos` sees (its last is `pos`)
-enum { MASK_CAUSAL = 0, MASK_WINDOW = 1, MASK_CHUNK = 2 };
+enum { MASK_CAUSAL = 0, MASK_WINDOW = 1, MASK_CHUNK = 2 };      // == tgx_mask (include/tgx.h)
 __device__ __forceinline__ int first_key(int pos, int kind, int size) {
   return kind == MASK_WINDOW ? max(0, pos - size + 1) : kind == MASK_CHUNK ? pos - pos % size : 0;
 }

@@ -89,18 +89,72 @@ static bool load_modepel_layer(const Json& L, size_t i, tgx_layer_desc& l, std::
   return true;
 }
 
+// the attention entries of a Vitudra mixer (an "attention" layer's, or the "left" half of a "parallel" one); what is absent is off
+static void load_vitudra_attention(const Json& m, int mask_kind, tgx_layer_desc& l) {
+  auto dim = [](const Json& j, const char* key) -> int32_t { const int64_t v = j.get_int(key, -1); return (v < 0 || v > ((int64_t)1 << 30)) ? -1 : (int32_t)v; };
+  l.heads = dim(m, "heads"); l.kv_heads = m.has("kv_heads") ? dim(m, "kv_heads") : l.heads; l.dim = dim(m, "dim"); l.vdim = m.has("vdim") ? dim(m, "vdim") : l.dim;
+  l.scale = m.get_float("scale", 1.f); l.softcap = m.get_float("softcap", 0.f);
+  const Json* mask = m.get("mask");
+  if (mask && mask->kind == Json::Obj) { l.mask_kind = mask_kind; l.mask_size = dim(*mask, "size"); }
+  const Json* rot = m.get("rot");
+  if (rot && rot->kind == Json::Obj) {
+    l.rot_dims = dim(*rot, "dims"); l.rot_base = rot->get_float("base", 10000.f); l.rot_pairs = 1; l.rot_factor = 1.f;
+    const Json* sc = rot->get("scaling");
+    if (sc && sc->kind == Json::Obj) l.rot_factor = sc->get_float("factor", 1.f);
+  }
+  const Json* qt = m.get("q_temp");
+  if (qt && qt->kind == Json::Obj) { l.q_temp_coef = qt->get_float("coef", 0.f); l.q_temp_every = dim(*qt, "every"); }
+}
+
+// one entry of a Vitudra config's "layers": {"type": "attention" | "wkv" | "parallel", "mixer": {...}, "mlp": null | {"kind": "dense", "ff"}}.  An attention
+// layer has a sliding window, a distance bias and a query temperature and may read another layer's keys and values ("kv_from"); a parallel mixer is
+// {"left": attention with neighbour-pair rotation, soft cap and chunked mask, "right": gated delta rule, "left_scale", "right_scale"}.  A wkv layer's decay
+// rank is left open: the device library takes it from the tensor's shape.
+static bool load_vitudra_layer(const Json& L, size_t i, tgx_layer_desc& l, std::string& err) {
+  auto dim = [](const Json& j, const char* key) -> int32_t { const int64_t v = j.get_int(key, -1); return (v < 0 || v > ((int64_t)1 << 30)) ? -1 : (int32_t)v; };
+  const Json* mx = L.get("mixer");
+  const Json* ff = L.get("mlp");
+  const std::string type = L.get_str("type", "");
+  auto bad = [&](const std::string& what) { err = "config.json: layer " + std::to_string(i) + ": " + what; return false; };
+  if (!mx || mx->kind != Json::Obj) return bad("no mixer");
+  if (type == "attention") {
+    l.mixer = TGX_MIXER_ATTENTION;
+    load_vitudra_attention(*mx, TGX_MASK_WINDOW, l);
+    l.dist_bias = 1;
+    if (mx->has("kv_from")) { const int32_t j = dim(*mx, "kv_from"); if (j < 0) return bad("kv_from"); l.kv_share = j + 1; }
+  } else if (type == "wkv") {
+    l.mixer = TGX_MIXER_WKV;
+    l.heads = dim(*mx, "heads"); l.dim = dim(*mx, "dim"); l.vdim = l.dim; l.kv_heads = l.heads;
+  } else if (type == "parallel") {
+    const Json* left = mx->get("left");
+    const Json* right = mx->get("right");
+    if (!left || left->kind != Json::Obj || !right || right->kind != Json::Obj) return bad("a parallel mixer needs left and right");
+    l.mixer = TGX_MIXER_PARALLEL;
+    load_vitudra_attention(*left, TGX_MASK_CHUNK, l);
+    l.d_heads = dim(*right, "heads"); l.d_kv_heads = right->has("kv_heads") ? dim(*right, "kv_heads") : l.d_heads; l.d_dim = dim(*right, "dim");
+    l.d_vdim = right->has("vdim") ? dim(*right, "vdim") : l.d_dim; l.conv_taps = right->has("conv") ? dim(*right, "conv") : 1;
+    l.left_scale = mx->get_float("left_scale", 1.f); l.right_scale = mx->get_float("right_scale", 1.f);
+  } else return bad("mixer '" + type + "' is not implemented");
+  if (!ff || ff->kind != Json::Obj) return true;
+  if (ff->get_str("kind", "") != "dense") return bad("feed-forward kind '" + ff->get_str("kind", "") + "' is not implemented");
+  l.mlp = TGX_MLP_DENSE; l.ff = dim(*ff, "ff");
+  return true;
+}
+
 // config.json of a layered model: {"architecture": "Zakusun", "width", "vocab", "logit_scale", "norm": {"eps", "groups"}, "canon": {"taps"},
 // "layers": [{"type": mixer, "mixer": {heads, dim, vdim, kv_rank, scale}, "mlp": null | {"kind": "moe", "expert": {ff, limit}, "router": {experts, top}}}]}
 // or {"architecture": "Modepel", "width", "vocab", "norm": {"eps"}, "layers": [...]} with the layer entries of load_modepel_layer
+// or {"architecture": "Vitudra", "width", "vocab", "residual_mult", "norm": {"eps"}, "layers": [...]} with the layer entries of load_vitudra_layer
 static bool load_stack_config(const Json& doc, const std::string& path, int compute_dtype, int max_batch, int max_ctx, int budget_tokens, ModelConfig& out, std::string& err) {
   const std::string arch = doc.get_str("architecture", "");
-  const bool modepel = arch == "Modepel";
+  const bool vitudra = arch == "Vitudra", modepel = arch == "Modepel" || vitudra;      // (both: scalar-free config header, a separate head)
   if (arch != "Zakusun" && !modepel) { err = "Unsupported architecture: " + arch; return false; }
   auto dim = [](const Json& j, const char* key) -> int32_t { const int64_t v = j.get_int(key, -1); return (v < 0 || v > ((int64_t)1 << 30)) ? -1 : (int32_t)v; };
   out.layered = true;
-  out.model_type = modepel ? "modepel" : "zakusun";
+  out.model_type = vitudra ? "vitudra" : modepel ? "modepel" : "zakusun";
   tgx_stack_desc& s = out.stack;
-  s.family = modepel ? TGX_FAMILY_MODEPEL : TGX_FAMILY_ZAKUSUN;
+  s.family = vitudra ? TGX_FAMILY_VITUDRA : modepel ? TGX_FAMILY_MODEPEL : TGX_FAMILY_ZAKUSUN;
+  s.residual_mult = doc.get_float("residual_mult", 1.f);
   s.width = dim(doc, "width"); s.vocab = dim(doc, "vocab"); s.compute_dtype = compute_dtype;
   s.max_seqs = max_batch < 1 ? 1 : max_batch;
   s.max_ctx = max_ctx > 0 ? max_ctx : 4096;
@@ -118,7 +172,7 @@ static bool load_stack_config(const Json& doc, const std::string& path, int comp
     const Json& L = layers->arr[i];
     tgx_layer_desc l{};
     if (modepel) {
-      if (!load_modepel_layer(L, i, l, err)) return false;
+      if (!(vitudra ? load_vitudra_layer(L, i, l, err) : load_modepel_layer(L, i, l, err))) return false;
       out.layers.push_back(l);
       continue;
     }
