@@ -83,7 +83,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--layered", default=None, metavar="SIZE[,SIZE]", help="instead of the headline: prefill and decode throughput of the layered (Zakusun) design at "
                     "layer sizes of real models (1b, 0.5b; random weights), beside a Llama-family model of the same width, depth and active parameters")
-    ap.add_argument("--design", default="zakusun", choices=["zakusun", "modepel"], help="with --layered: which layered design is measured beside the Llama-family model")
+    ap.add_argument("--only", default="", help="with --layered: measure these models only (names before the size, with commas; for profiling one of them)")
+    ap.add_argument("--design", default="zakusun", choices=["zakusun", "modepel", "vitudra"], help="with --layered: which layered design is measured beside its closest relatives and the Llama-family model")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample")
     return ap.parse_args()
 
@@ -332,6 +333,29 @@ def modepel_desc(key, z, L, V, dtype, B, ctx):
     return StackDesc(family="modepel", width=W, vocab=V, compute_dtype=dtype, max_seqs=B, max_ctx=ctx, budget_tokens=B * (ctx + 64), norm_eps=1e-5, name=f"modepel-{key}", layers=layers)
 
 
+def vitudra_desc(key, z, L, V, dtype, B, ctx):
+    """Vitudra at the size of `z`: wkv, parallel (chunked rotary attention beside a gated delta rule) and sliding-window attention layers in turn, every second
+    attention layer reading the keys and values of the one before; a gated feed-forward as wide as the Llama-family model's beside every mixer"""
+    from tinygpt_amd.desc import LayerDesc, StackDesc
+    W = z["width"]
+    layers, last_attn = [], None
+    for i in range(L):
+        if i % 3 == 0:
+            l = LayerDesc(mixer="wkv", heads=W // 64, kv_heads=W // 64, dim=64, vdim=64, decay_rank=64)
+        elif i % 3 == 1:
+            l = LayerDesc(mixer="parallel", heads=W // 128, kv_heads=max(1, W // 512), dim=128, vdim=128, scale=128 ** -0.5, rot_dims=32, rot_base=10000.0, rot_pairs=True,
+                          rot_factor=4.0, softcap=30.0, mask="chunk", mask_size=1024, d_heads=W // 128, d_kv_heads=max(1, W // 256), d_dim=128, d_vdim=128, conv_taps=4,
+                          left_scale=0.7, right_scale=1.1)
+        else:
+            l = LayerDesc(mixer="attention", heads=W // 128, kv_heads=max(1, W // 512), dim=128, vdim=128, scale=128 ** -0.5, mask="window", mask_size=1024, dist_bias=True,
+                          q_temp_coef=0.2, q_temp_every=128, kv_from=last_attn)
+            last_attn = i if last_attn is None else None
+        l.mlp, l.ff = "dense", z["top"] * z["ff"]
+        layers.append(l)
+    return StackDesc(family="vitudra", width=W, vocab=V, compute_dtype=dtype, max_seqs=B, max_ctx=ctx, budget_tokens=B * (ctx + 64), norm_eps=1e-5, residual_mult=0.5,
+                     name=f"vitudra-{key}", layers=layers)
+
+
 def layered_compare(args):
     from tinygpt_amd.desc import LayerDesc, ModelDesc, StackDesc
     from tinygpt_amd.ffi import GREEDY, Model
@@ -377,7 +401,11 @@ def layered_compare(args):
                                          top=z["top"], ff=z["ff"], limit=7.0) for _ in range(L)])
         ld = ModelDesc(family="llama", hidden=z["width"], layers=L, heads=z["llama"]["heads"], kv_heads=z["llama"]["kv_heads"], head_dim=z["width"] // z["llama"]["heads"],
                        inter=z["llama"]["inter"], vocab=V, max_ctx=ctx, tied=True, compute_dtype=args.dtype, norm_eps=1e-5, rope_theta=500000.0, max_batch=B, name=f"llama-{key}")
-        for desc, layered in ([(modepel_desc(key, z, L, V, args.dtype, B, ctx), True)] if args.design == "modepel" else []) + [(sd, True), (ld, False)]:
+        todo = {"zakusun": [(sd, True)], "modepel": [(modepel_desc(key, z, L, V, args.dtype, B, ctx), True), (sd, True)],
+                "vitudra": [(vitudra_desc(key, z, L, V, args.dtype, B, ctx), True), (modepel_desc(key, z, L, V, args.dtype, B, ctx), True)]}[args.design] + [(ld, False)]
+        if args.only:
+            todo = [t for t in todo if t[0].name.split("-")[0] in args.only.split(",")]
+        for desc, layered in todo:
             m = Model(desc).load_synthetic(1234, 0.02).finalize()
             r = measure(m, layered)
             m.close()

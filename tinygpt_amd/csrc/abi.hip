@@ -1243,7 +1243,8 @@ int tgx_set_option(tgx_ctx* c, const char* key, int value) {
   static const char* cls_names[TGX_KERNEL_COUNT] = {"qkv", "attn", "oproj", "gateup", "down", "lmhead"};
   if (c->stack) {      // layered models: "act.round16" as for the other families; "attn.split_min" = context from which steps of few tokens divide a sequence's keys
     if (!strcmp(key, "act.round16")) { c->act16 = value != 0; return TGX_OK; }      // between workgroups; "stack.gemm_wt" forces the product tile (1 / 2, 0 = automatic)
-    if (!strcmp(key, "attn.split_min")) { c->stack->attn_split_min_keys = value; return TGX_OK; }
+    if (!strcmp(key, "attn.split_min")) { c->stack->attn_split_min_keys = value; c->stack->gqa_split_min_keys = value; return TGX_OK; }
+    if (!strcmp(key, "attn.gqa_split_min")) { c->stack->gqa_split_min_keys = value; return TGX_OK; }
     if (!strcmp(key, "attn.mfma")) { c->stack->attn_mfma = value != 0; return TGX_OK; }      // 0: the lane-per-channel attention kernels for every layer
     if (!strcmp(key, "mlstm.narrow")) { c->stack->mlstm_narrow = value < 0 ? -1 : (value != 0); return TGX_OK; }      // the matrix-memory scan's column split (-1: automatic)
     if (!strcmp(key, "stack.gemv")) { c->stack->gemv = value != 0; return TGX_OK; }      // 0: products of few rows on the matrix-core tiles too

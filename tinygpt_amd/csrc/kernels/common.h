@@ -196,13 +196,13 @@ __device__ __forceinline__ float group_max(float v) {
   return v;
 }
 
-// Sum over aligned groups of 8 or 16 adjacent lanes on the DPP crossbar; every lane of the group gets the sum.
+// Sum over aligned groups of 4, 8 or 16 adjacent lanes on the DPP crossbar; every lane of the group gets the sum.
 template <int WIDTH>
 __device__ __forceinline__ float row_group_sum(float v) {
-  static_assert(WIDTH == 8 || WIDTH == 16, "row_group_sum: 8 or 16 lanes");
+  static_assert(WIDTH == 4 || WIDTH == 8 || WIDTH == 16, "row_group_sum: 4, 8 or 16 lanes");
   v += dpp_mov<0xB1, 0xf>(v);    // quad_perm:[1,0,3,2]
   v += dpp_mov<0x4E, 0xf>(v);    // quad_perm:[2,3,0,1]
-  v += dpp_mov<0x141, 0xf>(v);   // row_half_mirror
+  if (WIDTH >= 8) v += dpp_mov<0x141, 0xf>(v);   // row_half_mirror
   if (WIDTH == 16) v += dpp_mov<0x140, 0xf>(v);   // row_mirror
   return v;
 }

@@ -25,9 +25,9 @@ __global__ __launch_bounds__(256) void offset_norm_kernel(const float* x, const 
   for (int c = threadIdx.x; c < W; c += 256) out[(size_t)blockIdx.x * W + c] = xr[c] * r * (offset + w[c]);
 }
 
-// ---- token shift.  One workgroup per token: out[t][s] = h_t + (h_(t-1) - h_t) * mu[s] for the n mixes; h_(t-1) is the row before in the entry, the
-// slot's kept row for an entry's first token, zero at position 0.  The kept row is double-buffered with the slot's step parity (the entry's last token
-// writes buffer par ^ 1 while its first reads buffer par).
+// ---- token shift.  One thread per (token, channel): out[t][s] = h_t + (h_(t-1) - h_t) * mu[s] for the n mixes; h_(t-1) is the row before in the entry,
+// the slot's kept row for an entry's first token, zero at position 0.  The kept row is double-buffered with the slot's step parity (the entry's last
+// token writes buffer par ^ 1 while its first reads buffer par).  Grid: (tokens, width / 256).
 struct TokenShiftArgs {
   const float* h;        // [T][W]
   const float* mu;       // [n][W]
@@ -37,22 +37,22 @@ struct TokenShiftArgs {
   int W, n;
 };
 __global__ __launch_bounds__(256) void token_shift_kernel(StepMeta m, TokenShiftArgs a) {
-  const int t = blockIdx.x, i = m.tok_idx[t], cnt = m.tok_cnt[t], pos = m.tok_pos[t], row = m.tok_row[t], par = m.tok_par[t];
-  const float* cur = a.h + (size_t)t * a.W;
-  const float* before = i > 0 ? cur - a.W : a.state + (size_t)par * a.state_buf + (size_t)row * a.W;
-  const bool none = pos == 0;
-  float* keep = i == cnt - 1 ? a.state + (size_t)(par ^ 1) * a.state_buf + (size_t)row * a.W : nullptr;
-  for (int c = threadIdx.x; c < a.W; c += 256) {
-    const float x = cur[c], d = (none ? 0.f : before[c]) - x;
-    for (int s = 0; s < a.n; s++) a.out[((size_t)t * a.n + s) * a.W + c] = fmaf(d, a.mu[(size_t)s * a.W + c], x);
-    if (keep) keep[c] = x;
-  }
+  const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= a.W) return;
+  const int i = m.tok_idx[t], cnt = m.tok_cnt[t], pos = m.tok_pos[t], row = m.tok_row[t], par = m.tok_par[t];
+  const float* __restrict__ cur = a.h + (size_t)t * a.W;
+  const float* __restrict__ before = i > 0 ? cur - a.W : a.state + (size_t)par * a.state_buf + (size_t)row * a.W;
+  float* __restrict__ outp = a.out + (size_t)t * a.n * a.W;
+  const float x = cur[c], d = (pos == 0 ? 0.f : before[c]) - x;
+  for (int s = 0; s < a.n; s++) outp[(size_t)s * a.W + c] = fmaf(d, a.mu[(size_t)s * a.W + c], x);
+  if (i == cnt - 1) a.state[(size_t)(par ^ 1) * a.state_buf + (size_t)row * a.W + c] = x;
 }
 
-// ---- inputs of a gated-delta-rule layer.  One workgroup per token.  proj row = [.. | q (G D) | k (G D) | v (H E) | b (H) | a (H) | ..] from column col0;
-// the C = 2 G D + H E convolved channels take taps weights each (last = the current token's); the taps - 1 rows before come from the step's own rows, the
-// slot's tails (raw projections, double-buffered by step parity like the other per-slot rows) or are zero before the sequence's start.
+// ---- inputs of a gated-delta-rule layer.  proj row = [.. | q (G D) | k (G D) | v (H E) | b (H) | a (H) | ..] from column col0; the C = 2 G D + H E
+// convolved channels take taps weights each (last = the current token's); the taps - 1 rows before come from the step's own rows, the slot's tails (raw
+// projections, double-buffered by step parity like the other per-slot rows) or are zero before the sequence's start.
 // out row = [q | k | v | beta | decay]: q, k unit vectors per head (x / sqrt(sum x^2 + unit_eps)), q times q_scale.
+// Grid: (tokens, 2 G + H + 1): one workgroup per q head, k head (D <= 256 channels, one per thread, and their norm), v head, and one for the H gates.
 struct DeltaPrepArgs {
   const float* proj; long long ldp; int col0;
   const float* cw;       // [C][taps]
@@ -65,24 +65,38 @@ struct DeltaPrepArgs {
   float q_scale, unit_eps;
 };
 __global__ __launch_bounds__(256) void delta_prep_kernel(StepMeta m, DeltaPrepArgs a) {
-  extern __shared__ float s_c[];      // [C] the token's convolved, activated channels
-  const int t = blockIdx.x, i = m.tok_idx[t], cnt = m.tok_cnt[t], pos = m.tok_pos[t], row = m.tok_row[t], par = m.tok_par[t];
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int GD = a.kv_heads * a.dim, C = 2 * GD + a.heads * a.vdim, nb = a.taps - 1;
+  __shared__ float s4[4];
+  const int t = blockIdx.x, u = blockIdx.y, i = m.tok_idx[t], cnt = m.tok_cnt[t], pos = m.tok_pos[t], row = m.tok_row[t], par = m.tok_par[t];
+  const int G2 = 2 * a.kv_heads, GD = a.kv_heads * a.dim, C = 2 * GD + a.heads * a.vdim, nb = a.taps - 1;
   const float* __restrict__ pr = a.proj + (size_t)t * a.ldp + a.col0;
+  float* __restrict__ o = a.out + (size_t)t * a.ldo;
+  if (u == G2 + a.heads) {
+    for (int h = threadIdx.x; h < a.heads; h += 256) {
+      const float zb = pr[C + h], za = pr[C + a.heads + h] + a.dt_bias[h];
+      const float sp = za > 20.f ? za : log1pf(expf(za));
+      o[C + h] = 1.0f / (1.0f + expf(-zb));
+      o[C + a.heads + h] = expf(-expf(a.a_log[h]) * sp);
+    }
+    return;
+  }
+  const bool qk = u < G2;
+  const int n = qk ? a.dim : a.vdim, c0 = qk ? u * a.dim : 2 * GD + (u - G2) * a.vdim;
   const float* __restrict__ st_old = a.state ? a.state + (size_t)par * a.state_buf + (size_t)row * nb * C : nullptr;
   float* __restrict__ st_new = a.state ? a.state + (size_t)(par ^ 1) * a.state_buf + (size_t)row * nb * C : nullptr;
-  float* __restrict__ o = a.out + (size_t)t * a.ldo;
-  for (int c = threadIdx.x; c < C; c += 256) {
+  const float* __restrict__ cw = a.cw;
+  float mine = 0.f;                                        // a q / k head's channel of this thread (D <= 256)
+  for (int cc = threadIdx.x; cc < n; cc += 256) {
+    const int c = c0 + cc;
     const float x0 = pr[c];
-    float acc = a.cw[(size_t)c * a.taps + nb] * x0;
+    float acc = cw[(size_t)c * a.taps + nb] * x0;
     for (int d = 1; d <= nb; d++) {                        // the row d positions back
       float xv = 0.f;
       if (d <= i) xv = pr[c - (long long)d * a.ldp];
       else if (pos - d >= 0) xv = st_old[(size_t)(nb - (d - i)) * C + c];      // tail slot s holds position past - nb + s, past = pos - i
-      acc = fmaf(a.cw[(size_t)c * a.taps + nb - d], xv, acc);
+      acc = fmaf(cw[(size_t)c * a.taps + nb - d], xv, acc);
     }
-    s_c[c] = acc / (1.0f + expf(-acc));
+    const float act = acc / (1.0f + expf(-acc));
+    if (qk) mine = act; else o[c] = act;
     if (st_new) {
       const int s = nb - (cnt - i);                        // row i of cnt lands in tail slot nb - (cnt - i) ...
       if (s >= 0) st_new[(size_t)s * C + c] = x0;
@@ -90,27 +104,16 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(StepMeta m, DeltaPrepAr
         for (int k = 0; k + cnt < nb; k++) st_new[(size_t)k * C + c] = (pos - (nb - cnt - k) >= 0) ? st_old[(size_t)(k + cnt) * C + c] : 0.f;
     }
   }
-  __syncthreads();
-  for (int hd = wv; hd < 2 * a.kv_heads; hd += 4) {        // q heads, then k heads: one wave each
-    const float* v = s_c + (size_t)hd * a.dim;
-    float ss = 0.f;
-    for (int c = lane; c < a.dim; c += 64) ss = fmaf(v[c], v[c], ss);
-    ss = wave_sum(ss);
-    const float r = (hd < a.kv_heads ? a.q_scale : 1.0f) / sqrtf(ss + a.unit_eps);
-    for (int c = lane; c < a.dim; c += 64) o[(size_t)hd * a.dim + c] = v[c] * r;
-  }
-  for (int c = 2 * GD + threadIdx.x; c < C; c += 256) o[c] = s_c[c];
-  for (int h = threadIdx.x; h < a.heads; h += 256) {
-    const float zb = pr[C + h], za = pr[C + a.heads + h] + a.dt_bias[h];
-    const float sp = za > 20.f ? za : log1pf(expf(za));
-    o[C + h] = 1.0f / (1.0f + expf(-zb));
-    o[C + a.heads + h] = expf(-expf(a.a_log[h]) * sp);
-  }
+  if (!qk) return;
+  const float ss = block_sum_256(mine * mine, s4);
+  const float r = (u < a.kv_heads ? a.q_scale : 1.0f) / sqrtf(ss + a.unit_eps);
+  if ((int)threadIdx.x < n) o[c0 + threadIdx.x] = mine * r;
 }
 
-// ---- the recurrences.  One workgroup per (entry, head, 64 value columns) walks the entry's tokens in order, TB at a time: the block's per-key-channel
-// inputs (three vectors of `dim`) and the workgroup's value columns are staged in LDS, then every lane updates its DPER rows of its column: a wave owns 16
-// columns, its lanes = 4 row groups x 16 columns, 4 DPER >= dim.  Sums over the key channels cross the row groups by two lane exchanges.
+// ---- the recurrences.  One workgroup per (entry, head, 32 value columns) walks the entry's tokens in order, TB at a time: the block's per-key-channel
+// inputs (up to three vectors of `dim`) and the workgroup's value columns are staged in LDS (the next block's travel in registers meanwhile), then every
+// lane updates its DPER rows of its column with no barrier inside the block: a wave owns 8 columns, its lanes = 8 columns x 8 row groups (the row groups
+// of a column are adjacent lanes), 8 DPER >= dim.  Sums over the key channels cross the row groups on the lane crossbar.
 enum { REC_WKV = 0, REC_DELTA = 1 };
 struct RecScanArgs {
   const float* a; long long lda;     // per token and key head [dim]: the read vector (wkv: r, delta: q)
@@ -123,13 +126,15 @@ struct RecScanArgs {
   float* out; long long ldo;         // [T][heads * vdim]
   int heads, kv_heads, dim, vdim;
 };
+constexpr int REC_RG = 8, REC_COLS = 4 * (64 / REC_RG);      // row groups per column; columns per workgroup
 template <int DPER, int KIND>
 __global__ __launch_bounds__(256) void rec_scan_kernel(StepMeta m, RecScanArgs a) {
-  constexpr int LP = DPER + 4, DP = 4 * DPER, TB = DP <= 128 ? 16 : 8;      // LP: a row group's LDS stride (the groups' reads fall into different banks)
-  __shared__ __attribute__((aligned(16))) float s_a[TB][4 * LP], s_k[TB][4 * LP], s_w[KIND == REC_WKV ? TB : 1][4 * LP];
-  __shared__ float s_v[TB][64], s_b[TB], s_g[TB];
-  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, rg = lane >> 4, cl = lane & 15;
-  const int jl = wv * 16 + cl, j = blockIdx.z * 64 + jl;
+  constexpr int RG = REC_RG, CW = 64 / RG, CB = REC_COLS, LP = DPER + 4, DP = RG * DPER, TB = DP <= 128 ? 16 : 8;      // LP: a row group's LDS stride (the groups' reads fall into different banks)
+  constexpr int NQ = TB * DP / 256, NV = (TB * CB + 255) / 256, NA = KIND == REC_WKV ? 3 : 2;
+  __shared__ __attribute__((aligned(16))) float s_in[NA][TB][RG * LP];      // [0]: the read vector, [1]: k, [2]: the decay
+  __shared__ float s_v[TB][CB], s_b[TB], s_g[TB];
+  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, rg = lane % RG, cl = lane / RG;
+  const int jl = wv * CW + cl, j = blockIdx.z * CB + jl;
   const int start = m.ent_start[e], cnt = m.ent_count[e], row = m.ent_row[e];
   const bool fresh = m.tok_pos[start] == 0;
   const int kh = h / (a.heads / a.kv_heads), d0 = rg * DPER, l0 = rg * LP;
@@ -142,30 +147,49 @@ __global__ __launch_bounds__(256) void rec_scan_kernel(StepMeta m, RecScanArgs a
     S[dd] = (!fresh && d < a.dim && col) ? Sg[(size_t)d * a.vdim + j] : 0.f;
     if (KIND == REC_WKV) ub[dd] = d < a.dim ? a.u[(size_t)h * a.dim + d] : 0.f;
   }
+  const float* src[3] = {a.a, a.k, a.w};
+  const long long lds[3] = {a.lda, a.ldk, a.ldw};
+  float rin[NA][NQ], rv[NV], rb = 0.f, rgt = 0.f;
+  auto fetch = [&](int t0) {
+    const int nb = min(TB, cnt - t0);
+#pragma unroll
+    for (int u = 0; u < NQ; u++) {
+      const int i = tid + 256 * u, t = i / DP, d = i - t * DP;
+      const bool on = t < nb && d < a.dim;
+      const size_t tok = (size_t)(start + t0 + min(t, nb - 1));
+#pragma unroll
+      for (int s = 0; s < NA; s++) rin[s][u] = on ? src[s][tok * lds[s] + (size_t)kh * a.dim + d] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < NV; u++) {
+      const int i = tid + 256 * u, t = i / CB, c = i - t * CB;
+      rv[u] = (t < nb && blockIdx.z * CB + c < a.vdim) ? a.v[(size_t)(start + t0 + t) * a.ldv + (size_t)h * a.vdim + blockIdx.z * CB + c] : 0.f;
+    }
+    if (KIND == REC_DELTA && tid < nb) { rb = a.beta[(size_t)(start + t0 + tid) * a.ldg + h]; rgt = a.g[(size_t)(start + t0 + tid) * a.ldg + h]; }
+  };
+  fetch(0);
   for (int t0 = 0; t0 < cnt; t0 += TB) {
     const int nb = min(TB, cnt - t0);
     __syncthreads();                                       // the block before has been read
-    for (int i = tid; i < nb * DP; i += 256) {
-      const int t = i / DP, d = i - t * DP, at = (d / DPER) * LP + d % DPER;
-      const size_t tok = (size_t)(start + t0 + t);
-      const bool on = d < a.dim;
-      s_a[t][at] = on ? a.a[tok * a.lda + (size_t)kh * a.dim + d] : 0.f;
-      s_k[t][at] = on ? a.k[tok * a.ldk + (size_t)kh * a.dim + d] : 0.f;
-      if (KIND == REC_WKV) s_w[t][at] = on ? a.w[tok * a.ldw + (size_t)kh * a.dim + d] : 0.f;
+#pragma unroll
+    for (int u = 0; u < NQ; u++) {
+      const int i = tid + 256 * u, t = i / DP, d = i - t * DP, at = (d / DPER) * LP + d % DPER;
+#pragma unroll
+      for (int s = 0; s < NA; s++) s_in[s][t][at] = rin[s][u];
     }
-    for (int i = tid; i < nb * 64; i += 256) {
-      const int t = i >> 6, c = i & 63;
-      s_v[t][c] = blockIdx.z * 64 + c < a.vdim ? a.v[(size_t)(start + t0 + t) * a.ldv + (size_t)h * a.vdim + blockIdx.z * 64 + c] : 0.f;
-    }
-    if (KIND == REC_DELTA && tid < nb) { s_b[tid] = a.beta[(size_t)(start + t0 + tid) * a.ldg + h]; s_g[tid] = a.g[(size_t)(start + t0 + tid) * a.ldg + h]; }
+#pragma unroll
+    for (int u = 0; u < NV; u++) { const int i = tid + 256 * u; if (i < TB * CB) s_v[i / CB][i % CB] = rv[u]; }
+    if (KIND == REC_DELTA && tid < TB) { s_b[tid] = rb; s_g[tid] = rgt; }
     __syncthreads();
+    if (t0 + TB < cnt) fetch(t0 + TB);
     for (int t = 0; t < nb; t++) {
       const float vj = s_v[t][jl];
       float po = 0.f;
       if (KIND == REC_WKV) {
 #pragma unroll
         for (int dd = 0; dd < DPER; dd += 4) {
-          const f32x4 r4 = *reinterpret_cast<const f32x4*>(&s_a[t][l0 + dd]), k4 = *reinterpret_cast<const f32x4*>(&s_k[t][l0 + dd]), w4 = *reinterpret_cast<const f32x4*>(&s_w[t][l0 + dd]);
+          const f32x4 r4 = *reinterpret_cast<const f32x4*>(&s_in[0][t][l0 + dd]), k4 = *reinterpret_cast<const f32x4*>(&s_in[1][t][l0 + dd]),
+                      w4 = *reinterpret_cast<const f32x4*>(&s_in[NA - 1][t][l0 + dd]);
 #pragma unroll
           for (int q = 0; q < 4; q++) {
             const float kv = k4[q] * vj;
@@ -175,23 +199,24 @@ __global__ __launch_bounds__(256) void rec_scan_kernel(StepMeta m, RecScanArgs a
         }
       } else {
         const float g = s_g[t];
+        f32x4 kk[DPER / 4];
         float pk = 0.f;
 #pragma unroll
         for (int dd = 0; dd < DPER; dd += 4) {
-          const f32x4 k4 = *reinterpret_cast<const f32x4*>(&s_k[t][l0 + dd]);
+          kk[dd / 4] = *reinterpret_cast<const f32x4*>(&s_in[1][t][l0 + dd]);
 #pragma unroll
-          for (int q = 0; q < 4; q++) { S[dd + q] *= g; pk = fmaf(S[dd + q], k4[q], pk); }
+          for (int q = 0; q < 4; q++) { S[dd + q] *= g; pk = fmaf(S[dd + q], kk[dd / 4][q], pk); }
         }
-        pk += __shfl_xor(pk, 16, 64); pk += __shfl_xor(pk, 32, 64);
+        pk = row_group_sum<RG>(pk);
         const float uj = s_b[t] * (vj - pk);
 #pragma unroll
         for (int dd = 0; dd < DPER; dd += 4) {
-          const f32x4 k4 = *reinterpret_cast<const f32x4*>(&s_k[t][l0 + dd]), q4 = *reinterpret_cast<const f32x4*>(&s_a[t][l0 + dd]);
+          const f32x4 q4 = *reinterpret_cast<const f32x4*>(&s_in[0][t][l0 + dd]);
 #pragma unroll
-          for (int q = 0; q < 4; q++) { S[dd + q] = fmaf(k4[q], uj, S[dd + q]); po = fmaf(S[dd + q], q4[q], po); }
+          for (int q = 0; q < 4; q++) { S[dd + q] = fmaf(kk[dd / 4][q], uj, S[dd + q]); po = fmaf(S[dd + q], q4[q], po); }
         }
       }
-      po += __shfl_xor(po, 16, 64); po += __shfl_xor(po, 32, 64);
+      po = row_group_sum<RG>(po);
       if (rg == 0 && col) a.out[(size_t)(start + t0 + t) * a.ldo + (size_t)h * a.vdim + j] = po;
     }
   }

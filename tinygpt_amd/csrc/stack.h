@@ -83,6 +83,7 @@ struct StackModel {
   int *sel = nullptr, *moe_off = nullptr, *perm = nullptr, *ptok = nullptr, *tile_e = nullptr, *tile_m0 = nullptr, *n_tiles = nullptr;
   int max_in = 0, max_hr = 0, max_hv = 0, max_top = 0, max_ff = 0, max_E = 0, max_rank = 0;
   int attn_split_min_keys = 2048;      // option attn.split_min: steps of few tokens split a sequence's keys between workgroups from this context on
+  int gqa_split_min_keys = 1024;       // option attn.gqa_split_min: the same threshold for the grouped-query kernels, counted in keys a workgroup would walk (a mask's span); attn.split_min sets both
   int attn_mfma = 1;                   // option attn.mfma: 0 keeps every layer on the lane-per-channel attention kernels
   int gemv = 1;                        // option stack.gemv: 0 sends products of few rows through the matrix-core tiles as well
   int mlstm_narrow = -1;               // option mlstm.narrow: the matrix-memory scan's columns per wave (1: eight, 0: sixteen, -1: by the step's entries and heads)

@@ -371,7 +371,7 @@ int run_gqa_core(tgx_ctx* c, const tgx::StepMeta& m, const GqaSpec& sp, int T, i
     const int tiles = (max_count * (H / G) + 31) / 32;
     const long long wgs = (long long)tiles * S * G;
     int nsplit = 1;
-    if (span >= sm->attn_split_min_keys && wgs < c->num_cus) {
+    if (span >= sm->gqa_split_min_keys && wgs < c->num_cus) {
       nsplit = (int)std::min<long long>(64, (2LL * c->num_cus) / wgs);
       const int per = std::max(64, ((span + nsplit - 1) / nsplit + 63) / 64 * 64);      // whole key tiles
       nsplit = (span + per - 1) / per;
@@ -395,7 +395,7 @@ int run_gqa_core(tgx_ctx* c, const tgx::StepMeta& m, const GqaSpec& sp, int T, i
   aa.heads = H; aa.kv_heads = G; aa.dim = sp.dim; aa.vdim = sp.vdim; aa.scale = sp.scale; aa.sink = sp.sink; aa.has_sink = sp.has_sink;
   aa.mask_kind = sp.mask_kind; aa.mask_size = sp.mask_size; aa.softcap = sp.softcap; aa.dist_bias = sp.dist_bias;
   int nsplit = 1;
-  if (span >= sm->attn_split_min_keys && (long long)T * H < 2LL * c->num_cus) {      // few (token, head) pairs and a long context: the keys are divided between workgroups
+  if (span >= sm->gqa_split_min_keys && (long long)T * H < 2LL * c->num_cus) {      // few (token, head) pairs and a long context: the keys are divided between workgroups
     nsplit = (int)std::min<long long>(64, (4LL * c->num_cus) / ((long long)T * H));
     const int per = std::max(256, ((span + nsplit - 1) / nsplit + 63) / 64 * 64);
     nsplit = (span + per - 1) / per;
@@ -566,14 +566,14 @@ void add_to_stream(tgx_ctx* c, const float* A, int K, const ebyte* Wm, int T, fl
 }
 
 void launch_rec_scan(tgx_ctx* c, const tgx::StepMeta& m, const tgx::RecScanArgs& a, int kind, int S) {
-  const dim3 grid(S, a.heads, (a.vdim + 63) / 64);
-  const int dper = (a.dim + 3) / 4;
+  const dim3 grid(S, a.heads, (a.vdim + tgx::REC_COLS - 1) / tgx::REC_COLS);
+  const int dper = (a.dim + tgx::REC_RG - 1) / tgx::REC_RG;      // rows per lane
   auto go = [&](auto K) {
     constexpr int KIND = decltype(K)::value;
-    if (dper <= 8) hipLaunchKernelGGL((tgx::rec_scan_kernel<8, KIND>), grid, dim3(256), 0, c->stream, m, a);
+    if (dper <= 4) hipLaunchKernelGGL((tgx::rec_scan_kernel<4, KIND>), grid, dim3(256), 0, c->stream, m, a);
+    else if (dper <= 8) hipLaunchKernelGGL((tgx::rec_scan_kernel<8, KIND>), grid, dim3(256), 0, c->stream, m, a);
     else if (dper <= 16) hipLaunchKernelGGL((tgx::rec_scan_kernel<16, KIND>), grid, dim3(256), 0, c->stream, m, a);
-    else if (dper <= 32) hipLaunchKernelGGL((tgx::rec_scan_kernel<32, KIND>), grid, dim3(256), 0, c->stream, m, a);
-    else hipLaunchKernelGGL((tgx::rec_scan_kernel<64, KIND>), grid, dim3(256), 0, c->stream, m, a);
+    else hipLaunchKernelGGL((tgx::rec_scan_kernel<32, KIND>), grid, dim3(256), 0, c->stream, m, a);
   };
   if (kind == tgx::REC_WKV) go(std::integral_constant<int, tgx::REC_WKV>{}); else go(std::integral_constant<int, tgx::REC_DELTA>{});
 }
@@ -603,7 +603,7 @@ void run_wkv(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, int T, int S) {
   const int W = sm->d.width, H = ld.heads, HD = H * ld.dim, R = ld.decay_rank;
   tgx::TokenShiftArgs ts{};
   ts.h = sm->a; ts.mu = w.mu; ts.out = sm->mixed; ts.state = w.shift; ts.state_buf = (size_t)sm->d.max_seqs * W; ts.W = W; ts.n = 5;
-  hipLaunchKernelGGL(tgx::token_shift_kernel, dim3(T), dim3(256), 0, c->stream, m, ts);
+  hipLaunchKernelGGL(tgx::token_shift_kernel, dim3(T, (W + 255) / 256), dim3(256), 0, c->stream, m, ts);
   // proj row = [r | k | v | g | w]: the first four as one product batched over their mixes, the decay through its low-rank pair
   tgx::StackGemmArgs g{};
   g.A = sm->mixed; g.lda = 5LL * W; g.a_zoff = W; g.B = w.w_in; g.ldb = W; g.b_zstride = (long long)HD * W; g.C = sm->proj; g.ldc = 5LL * HD; g.c_zoff = HD;
@@ -649,7 +649,7 @@ int run_parallel(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, int T, int 
   dp.proj = sm->proj; dp.ldp = nin; dp.col0 = lq + lkv; dp.cw = w.conv_w; dp.a_log = w.a_log; dp.dt_bias = w.dt_bias; dp.out = sm->rec_in; dp.ldo = ldr;
   dp.state = nb > 0 ? w.conv_state : nullptr; dp.state_buf = (size_t)sm->d.max_seqs * nb * rC; dp.heads = rH; dp.kv_heads = rG; dp.dim = ld.d_dim; dp.vdim = ld.d_vdim; dp.taps = ld.conv_taps;
   dp.q_scale = 1.0f / sqrtf((float)ld.d_dim); dp.unit_eps = 1e-6f;
-  hipLaunchKernelGGL(tgx::delta_prep_kernel, dim3(T), dim3(256), (size_t)rC * 4, c->stream, m, dp);
+  hipLaunchKernelGGL(tgx::delta_prep_kernel, dim3(T, 2 * rG + rH + 1), dim3(256), 0, c->stream, m, dp);
   tgx::RecScanArgs ra{};
   ra.a = sm->rec_in; ra.lda = ldr; ra.k = sm->rec_in + rGD; ra.ldk = ldr; ra.v = sm->rec_in + 2 * (size_t)rGD; ra.ldv = ldr;
   ra.beta = sm->rec_in + rC; ra.g = sm->rec_in + rC + rH; ra.ldg = ldr; ra.S = w.mS; ra.out = sm->hs; ra.ldo = rvd; ra.heads = rH; ra.kv_heads = rG; ra.dim = ld.d_dim; ra.vdim = ld.d_vdim;
@@ -1088,7 +1088,6 @@ int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int d
         if (!attention_ok(why) || l.kv_share) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: parallel, attention half: %s", i, l.kv_share ? "shared keys are not part of it" : why);
         if (l.d_heads <= 0 || l.d_kv_heads <= 0 || l.d_heads % l.d_kv_heads || l.d_dim <= 0 || l.d_dim > 256 || l.d_vdim <= 0 || l.conv_taps < 1 || l.conv_taps > tgx::CONV_MAX_TAPS)
           return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: parallel, delta-rule half: %d heads over %d key heads of %d (1 .. 256) x %d, %d taps (1 .. %d)", i, l.d_heads, l.d_kv_heads, l.d_dim, l.d_vdim, l.conv_taps, tgx::CONV_MAX_TAPS);
-        if ((2LL * l.d_kv_heads * l.d_dim + (long long)l.d_heads * l.d_vdim) * 4 > 60000) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: parallel, delta-rule half: more than 15000 convolved channels", i);
       } else return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: mixer %d is not part of this family (attention, wkv and parallel are)", i, l.mixer);
       if (l.mlp != TGX_MLP_NONE && l.mlp != TGX_MLP_DENSE) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: feed-forward kind %d is not implemented", i, l.mlp);
       if (l.mlp == TGX_MLP_DENSE && l.ff <= 0) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: ff %d", i, l.ff);
