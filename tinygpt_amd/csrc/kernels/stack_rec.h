@@ -182,42 +182,45 @@ __global__ __launch_bounds__(256) void rec_scan_kernel(StepMeta m, RecScanArgs a
     if (KIND == REC_DELTA && tid < TB) { s_b[tid] = rb; s_g[tid] = rgt; }
     __syncthreads();
     if (t0 + TB < cnt) fetch(t0 + TB);
-    for (int t = 0; t < nb; t++) {
-      const float vj = s_v[t][jl];
+    // a token's operands travel from LDS to registers one token ahead of their use (two register sets, taken in turn), so the reads' latency lies under
+    // the arithmetic of the token before instead of on the recurrence's critical path
+    struct Tok { f32x4 in[NA][DPER / 4]; float v, g, b; };
+    auto take = [&](Tok& k, int t) {
+#pragma unroll
+      for (int s = 0; s < NA; s++)
+#pragma unroll
+        for (int dd = 0; dd < DPER; dd += 4) k.in[s][dd / 4] = *reinterpret_cast<const f32x4*>(&s_in[s][t][l0 + dd]);
+      k.v = s_v[t][jl];
+      if (KIND == REC_DELTA) { k.g = s_g[t]; k.b = s_b[t]; }
+    };
+    auto advance = [&](const Tok& k, int t) {
       float po = 0.f;
       if (KIND == REC_WKV) {
 #pragma unroll
-        for (int dd = 0; dd < DPER; dd += 4) {
-          const f32x4 r4 = *reinterpret_cast<const f32x4*>(&s_in[0][t][l0 + dd]), k4 = *reinterpret_cast<const f32x4*>(&s_in[1][t][l0 + dd]),
-                      w4 = *reinterpret_cast<const f32x4*>(&s_in[NA - 1][t][l0 + dd]);
-#pragma unroll
-          for (int q = 0; q < 4; q++) {
-            const float kv = k4[q] * vj;
-            po = fmaf(r4[q], fmaf(ub[dd + q], kv, S[dd + q]), po);
-            S[dd + q] = fmaf(w4[q], S[dd + q], kv);
-          }
+        for (int dd = 0; dd < DPER; dd++) {
+          const float kv = k.in[1][dd / 4][dd & 3] * k.v;
+          po = fmaf(k.in[0][dd / 4][dd & 3], fmaf(ub[dd], kv, S[dd]), po);
+          S[dd] = fmaf(k.in[NA - 1][dd / 4][dd & 3], S[dd], kv);
         }
       } else {
-        const float g = s_g[t];
-        f32x4 kk[DPER / 4];
         float pk = 0.f;
 #pragma unroll
-        for (int dd = 0; dd < DPER; dd += 4) {
-          kk[dd / 4] = *reinterpret_cast<const f32x4*>(&s_in[1][t][l0 + dd]);
-#pragma unroll
-          for (int q = 0; q < 4; q++) { S[dd + q] *= g; pk = fmaf(S[dd + q], kk[dd / 4][q], pk); }
-        }
+        for (int dd = 0; dd < DPER; dd++) { S[dd] *= k.g; pk = fmaf(S[dd], k.in[1][dd / 4][dd & 3], pk); }
         pk = row_group_sum<RG>(pk);
-        const float uj = s_b[t] * (vj - pk);
+        const float uj = k.b * (k.v - pk);
 #pragma unroll
-        for (int dd = 0; dd < DPER; dd += 4) {
-          const f32x4 q4 = *reinterpret_cast<const f32x4*>(&s_in[0][t][l0 + dd]);
-#pragma unroll
-          for (int q = 0; q < 4; q++) { S[dd + q] = fmaf(kk[dd / 4][q], uj, S[dd + q]); po = fmaf(S[dd + q], q4[q], po); }
-        }
+        for (int dd = 0; dd < DPER; dd++) { S[dd] = fmaf(k.in[1][dd / 4][dd & 3], uj, S[dd]); po = fmaf(S[dd], k.in[0][dd / 4][dd & 3], po); }
       }
       po = row_group_sum<RG>(po);
       if (rg == 0 && col) a.out[(size_t)(start + t0 + t) * a.ldo + (size_t)h * a.vdim + j] = po;
+    };
+    Tok ka, kb;
+    take(ka, 0);
+    for (int t = 0; t < nb; t += 2) {
+      take(kb, min(t + 1, TB - 1));
+      advance(ka, t);
+      take(ka, min(t + 2, TB - 1));
+      if (t + 1 < nb) advance(kb, t + 1);
     }
   }
 #pragma unroll
