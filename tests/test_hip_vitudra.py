@@ -106,6 +106,7 @@ MECH = {
     "one_tap": [par(right={"conv": 1})],
     "two_taps": [par(right={"conv": 2})],
     "eight_taps": [par(right={"conv": 8})],
+    "more_taps_than_tokens_in_a_page": [par(right={"conv": 30})],
     "delta_every_head_its_own_keys": [par(right={"heads": 3, "kv_heads": 3})],
     "delta_one_key_head": [par(right={"heads": 6, "kv_heads": 1})],
     "delta_wide_values": [par(right={"heads": 2, "kv_heads": 1, "dim": 12, "vdim": 70})],
@@ -447,7 +448,7 @@ def test_what_the_library_refuses():
                 [attn(kv_from=0)],                        # a layer cannot read its own (missing) pool
                 [wkv(), attn(kv_from=0)],                 # ... nor a layer without keys
                 [par(right={"heads": 4, "kv_heads": 3})],
-                [par(right={"conv": 9})],
+                [par(right={"conv": 65})],
                 [attn(mask={"size": 0})]):
         with pytest.raises(TgxError):
             Model(stack_desc_from_config(config(bad), "fp32"))

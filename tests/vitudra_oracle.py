@@ -128,7 +128,8 @@ def short_conv(x, w):
     out = np.zeros_like(x)
     for j in range(taps):
         back = taps - 1 - j
-        out[back:] += x[:T - back] * w[:, j] if back else x * w[:, j]
+        if back < T:
+            out[back:] += x[:T - back] * w[:, j]
     return out
 
 

@@ -53,6 +53,7 @@ __global__ __launch_bounds__(256) void token_shift_kernel(StepMeta m, TokenShift
 // projections, double-buffered by step parity like the other per-slot rows) or are zero before the sequence's start.
 // out row = [q | k | v | beta | decay]: q, k unit vectors per head (x / sqrt(sum x^2 + unit_eps)), q times q_scale.
 // Grid: (tokens, 2 G + H + 1): one workgroup per q head, k head (D <= 256 channels, one per thread, and their norm), v head, and one for the H gates.
+constexpr int DELTA_MAX_TAPS = 64;      // (bounds the per-slot tails, not the kernel: it loops over the taps)
 struct DeltaPrepArgs {
   const float* proj; long long ldp; int col0;
   const float* cw;       // [C][taps]

@@ -1086,8 +1086,8 @@ int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int d
         if (l.heads <= 0 || l.dim <= 0 || l.dim > 256 || l.decay_rank < 0) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: wkv: %d heads of %d (1 .. 256), decay rank %d", i, l.heads, l.dim, l.decay_rank);
       } else if (l.mixer == TGX_MIXER_PARALLEL) {
         if (!attention_ok(why) || l.kv_share) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: parallel, attention half: %s", i, l.kv_share ? "shared keys are not part of it" : why);
-        if (l.d_heads <= 0 || l.d_kv_heads <= 0 || l.d_heads % l.d_kv_heads || l.d_dim <= 0 || l.d_dim > 256 || l.d_vdim <= 0 || l.conv_taps < 1 || l.conv_taps > tgx::CONV_MAX_TAPS)
-          return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: parallel, delta-rule half: %d heads over %d key heads of %d (1 .. 256) x %d, %d taps (1 .. %d)", i, l.d_heads, l.d_kv_heads, l.d_dim, l.d_vdim, l.conv_taps, tgx::CONV_MAX_TAPS);
+        if (l.d_heads <= 0 || l.d_kv_heads <= 0 || l.d_heads % l.d_kv_heads || l.d_dim <= 0 || l.d_dim > 256 || l.d_vdim <= 0 || l.conv_taps < 1 || l.conv_taps > tgx::DELTA_MAX_TAPS)
+          return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: parallel, delta-rule half: %d heads over %d key heads of %d (1 .. 256) x %d, %d taps (1 .. %d)", i, l.d_heads, l.d_kv_heads, l.d_dim, l.d_vdim, l.conv_taps, tgx::DELTA_MAX_TAPS);
       } else return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: mixer %d is not part of this family (attention, wkv and parallel are)", i, l.mixer);
       if (l.mlp != TGX_MLP_NONE && l.mlp != TGX_MLP_DENSE) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: feed-forward kind %d is not implemented", i, l.mlp);
       if (l.mlp == TGX_MLP_DENSE && l.ff <= 0) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: ff %d", i, l.ff);
