@@ -27,8 +27,10 @@ extern "C" {
 
 /* 3 (round 5): per-row sequence lifecycle (tgx_reset_row / tgx_forward_row / tgx_sample_row / tgx_past_length_row); tgx_get_option added and
  * tgx_engine_read_stats + the options engine.*, pf.*, attn.fold_*, lmhead.fuse_finalize removed since 2. */
-#define TGX_ABI_VERSION 6   /* 4: layered models (tgx_create_stack, tgx_step_ragged); 5: Modepel (more mixers / feed-forward kinds in tgx_layer_desc);
-                             * 6: Vitudra (masks, score bias and cap, shared key / value layers, two recurrent mixers, parallel sublayers) */
+#define TGX_ABI_VERSION 7   /* 4: layered models (tgx_create_stack, tgx_step_ragged); 5: Modepel (more mixers / feed-forward kinds in tgx_layer_desc);
+                             * 6: Vitudra (masks, score bias and cap, shared key / value layers, two recurrent mixers, parallel sublayers);
+                             * 7: Zaluvik (layer norms around every sublayer, a looped span of layers, un-normalised sigmoid attention with mixed heads,
+                             *    windowed latent attention with a shared rotated key part, sigmoid group-limited router) */
 
 #if defined(__GNUC__)
 #define TGX_API __attribute__((visibility("default")))
@@ -59,8 +61,11 @@ typedef enum tgx_family {
   TGX_FAMILY_MISTRAL = 5,
   TGX_FAMILY_ZAKUSUN = 6,  /* a layered model (tgx_stack_desc below), no counterpart in the reference */
   TGX_FAMILY_MODEPEL = 7,  /* a layered model: rotary grouped-query attention and matrix-memory (mLSTM) layers, sandwich norms */
-  TGX_FAMILY_VITUDRA = 8   /* a layered model: one norm per layer in front of a mixer and a gated feed-forward that run side by side; windowed and chunked
+  TGX_FAMILY_VITUDRA = 8,  /* a layered model: one norm per layer in front of a mixer and a gated feed-forward that run side by side; windowed and chunked
                             * attention, shared key / value layers, decaying matrix states (token-shift "wkv" and gated delta rule) */
+  TGX_FAMILY_ZALUVIK = 9   /* a layered model: layer norms (weight and bias) before and after every sublayer, a span of layers run several times with the
+                            * embedding output fed back in, windowed sigmoid attention whose weights are mixed across heads, windowed latent attention
+                            * with a rotated key part all heads share, erf-gelu feed-forwards and sigmoid-routed experts; logits against the embedding table */
 } tgx_family;
 
 /* tinytorch::DType values the CLI accepts (examples/inference/main.cpp:82-88) */
@@ -134,7 +139,22 @@ typedef struct tgx_model_desc {
  *   gated delta rule          causal depth-wise convolutions of conv_taps taps and silu on q, k, v; unit q and k; S <- g S; S += k (beta (v - S^T k))^T;
  *                             o = S^T q; per-head unit norm, a weight shared by the heads, silu gate
  *   parallel mixer            left_scale * attention + right_scale * gated delta rule on the same input (the d_* fields size the right half)
- *   dense gated feed-forward  down(silu(gate h) * (up h)) */
+ *   dense gated feed-forward  down(silu(gate h) * (up h))
+ * and, for TGX_FAMILY_ZALUVIK (x <- x + residual_mult * LN_b(sublayer(LN_a(x))), LN(v) = (v - mean) / sqrt(var + norm_eps) * w + b; slots hold pages of one
+ * key / value pool (attention) or latent pool (latent attention) per layer RUN, so a layer inside the loop keeps one cache per pass):
+ *   embedding scale           x = embed[token] * embed_scale
+ *   loop                      layers loop_start .. loop_stop - 1 run loop_times times in a row with the same weights; in front of the first layer of every
+ *                             pass x <- W_loop [x; x0], x0 the embedding output ("loop.in" [width][2 width])
+ *   unit queries and keys     qk_norm 1: every query and key head is divided by sqrt(mean(head^2) + norm_eps) (no weight)
+ *   sigmoid attention         score_fn 1: the weight of a visible key is sigmoid(q . k * scale + pb[head]); weights are not normalised over the keys
+ *   mixed heads               head_mix 1: weight_h(i, j) <- sum_g talk[h][g] weight_g(i, j) before the values are summed (head h keeps its own value head)
+ *   output gates              gate_kind 1: per output channel, sigmoid(W_g h) [heads * vdim]; 2: per head, sigmoid(W_g h) [heads]
+ *   latent attention, rotated latent attention with rot_dim further query / key dimensions per head: the projection "dkv" has kv_rank + rot_dim rows, the last
+ *                             rot_dim of which (not normed, rotated by position, rotate-half pairing over rot_dims = rot_dim) are a key part all heads
+ *                             share; score = (q_plain . W_uk c + q_rot . k_rot) * scale; softmax without sink; mask_kind / mask_size as above
+ *   erf-gelu feed-forward     ff_act 1: down(gelu(up h)), gelu(z) = z (1 + erf(z / sqrt 2)) / 2
+ *   sigmoid router            router_fn 1: scores = sigmoid(W_r h) (32-bit), no correction; group_score 1: a group counts as the sum of its two largest
+ *                             scores; router_norm 1: weights = chosen scores / (their sum + 1e-20); a shared expert (shared_ff) without a gate of its own */
 typedef enum tgx_mixer { TGX_MIXER_LATENT_ATTENTION = 1, TGX_MIXER_ATTENTION = 2, TGX_MIXER_MLSTM = 3, TGX_MIXER_WKV = 4, TGX_MIXER_PARALLEL = 5 } tgx_mixer;
 typedef enum tgx_mlp { TGX_MLP_NONE = 0, TGX_MLP_MOE = 1, TGX_MLP_DENSE = 2 } tgx_mlp;
 typedef enum tgx_mask { TGX_MASK_CAUSAL = 0, TGX_MASK_WINDOW = 1, TGX_MASK_CHUNK = 2 } tgx_mask;
@@ -180,10 +200,20 @@ typedef struct tgx_layer_desc {
   int32_t conv_taps; /*           ... taps of its input convolutions                             */
   float left_scale;  /* parallel: weight of the attention half                                    */
   float right_scale; /* parallel: weight of the gated delta rule                                  */
+  /* ABI 7 (zero for the kinds that do not read them) */
+  int32_t qk_norm;   /* attention: 1 = unit-RMS queries and keys per head                         */
+  int32_t score_fn;  /* attention: 0 = softmax over the visible keys, 1 = sigmoid(score + per-head bias), not normalised */
+  int32_t head_mix;  /* attention: 1 = weights mixed across heads by a [heads][heads] matrix      */
+  int32_t gate_kind; /* output gate: 0 = the family's own, 1 = per channel, 2 = per head          */
+  int32_t rot_dim;   /* latent attention: rotated query / key dimensions per head beside `dim` (0: none) */
+  int32_t ff_act;    /* dense feed-forward: 0 = the family's own, 1 = erf gelu without a gate     */
+  int32_t router_fn; /* experts: 0 = softmax scores + correction, 1 = sigmoid scores              */
+  int32_t group_score; /* experts: a group counts as 0 = its largest, 1 = the sum of its two largest scores */
+  int32_t router_norm; /* experts: 1 = weights divided by their sum + 1e-20                       */
 } tgx_layer_desc;
 
 typedef struct tgx_stack_desc {
-  int32_t family;         /* tgx_family (TGX_FAMILY_ZAKUSUN, TGX_FAMILY_MODEPEL, TGX_FAMILY_VITUDRA) */
+  int32_t family;         /* tgx_family (TGX_FAMILY_ZAKUSUN, TGX_FAMILY_MODEPEL, TGX_FAMILY_VITUDRA, TGX_FAMILY_ZALUVIK) */
   int32_t width;          /* residual width                                                        */
   int32_t layers;         /* entries of the tgx_layer_desc array                                   */
   int32_t vocab;
@@ -196,7 +226,12 @@ typedef struct tgx_stack_desc {
   float norm_eps;
   int32_t canon_taps;     /* taps of the input convolution (>= 1)                                  */
   float logit_scale;      /* logits = embed . norm(x) * logit_scale                                */
-  float residual_mult;    /* ABI 6, TGX_FAMILY_VITUDRA: the factor on what a layer adds to the stream */
+  float residual_mult;    /* ABI 6, TGX_FAMILY_VITUDRA / ZALUVIK: the factor on what a sublayer adds to the stream */
+  /* ABI 7, TGX_FAMILY_ZALUVIK */
+  float embed_scale;      /* x = embed[token] * embed_scale                                         */
+  int32_t loop_start;     /* layers loop_start .. loop_stop - 1 run loop_times times (loop_times <= 1 or an empty span: no loop) */
+  int32_t loop_stop;
+  int32_t loop_times;
 } tgx_stack_desc;
 
 /* SamplerConfig (src/engine/Sampler.h:13-22).  Greedy iff temperature<=0 && top_k<=0 &&
@@ -223,7 +258,9 @@ TGX_API int tgx_create(const tgx_model_desc* desc, int device_ordinal, tgx_ctx**
  * TGX_FAMILY_MODEPEL: "embed", "head", "final.norm", "l<i>.norm1|norm1b|norm2|norm2b", attention "l<i>.mix.q|k|v(.b)|vmix|g|o", mLSTM
  * "l<i>.mix.q|k|v|g|o|norm|i(.b)|f(.b)", dense "l<i>.mlp.up|down|act", experts "l<i>.mlp.router|correction|e<j>.gate|up|down|shared.gate|up|down|sg".
  * TGX_FAMILY_VITUDRA: "embed", "head", "final.norm", "l<i>.norm1", "l<i>.mlp.gate|up|down", attention "l<i>.mix.q|k|v|o" (no k, v with kv_share), wkv
- * "l<i>.mix.mu.r|k|v|g|w", "l<i>.mix.r|k|v|g|w1|w2|w0|u|norm|o", parallel "l<i>.mix.left.q|k|v|o", "l<i>.mix.right.q|k|v(.conv)|b|a|A_log|dt_bias|g|norm|o". */
+ * "l<i>.mix.mu.r|k|v|g|w", "l<i>.mix.r|k|v|g|w1|w2|w0|u|norm|o", parallel "l<i>.mix.left.q|k|v|o", "l<i>.mix.right.q|k|v(.conv)|b|a|A_log|dt_bias|g|norm|o".
+ * TGX_FAMILY_ZALUVIK: "embed", "loop.in" (with a loop), "final.norm(.b)", "l<i>.norm1|norm1b|norm2|norm2b(.b)", attention "l<i>.mix.q|k|v|talk|pb|g|o", latent
+ * attention "l<i>.mix.q|dkv|dkv.norm|uk|uv|g|o", dense "l<i>.mlp.up|down", experts "l<i>.mlp.router|e<j>.gate|up|down|shared.gate|up|down". */
 TGX_API int tgx_create_stack(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int device_ordinal, tgx_ctx** out_ctx);
 
 /* == SafeTensors::loadInternal -> Storage::copyOnDevice for ONE named tensor

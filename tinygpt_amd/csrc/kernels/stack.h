@@ -159,6 +159,13 @@ struct LatentAppendArgs {
   void* pool;                                    // [pages][page][rank]
   void* poolT;                                   // [pages][rank][page]: the same latents, token-contiguous per channel (nullptr: not kept)
   int rank; float eps;
+  // a rotated key part all heads share (rot_dim > 0): the rot_dim columns behind the latent, not normed, turned by the token's position (rotate-half
+  // pairing over the first rot_dims of them, cosine / sine from a host-made table), are stored behind the normed latent: a pool row is [rank + rot_dim].
+  // The rotated part of every head's query (q columns [h * qstride + qoff, + rot_dim)) is turned the same way, multiplied by qscale and written behind
+  // the head's latent-space query: ql[t][h * (rank + rot_dim) + rank + i]
+  int rot_dim, rot_dims; const float* cs;        // cs [positions][rot_dims / 2][2]
+  const float* q; int heads, qstride, qoff; float qscale;
+  float* ql;
 };
 template <int DT>
 __global__ __launch_bounds__(64) void latent_append_kernel(StepMeta m, LatentAppendArgs a) {
@@ -169,12 +176,31 @@ __global__ __launch_bounds__(64) void latent_append_kernel(StepMeta m, LatentApp
   ss = wave_sum(ss);
   const float rinv = 1.0f / sqrtf(ss / (float)a.rank + a.eps);
   const int page = m.tbl[(size_t)m.tok_row[t] * m.tbl_stride + (pos >> m.page_shift)];
-  elem_t<DT>* dst = reinterpret_cast<elem_t<DT>*>(a.pool) + (((size_t)page << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1))) * a.rank;
-  elem_t<DT>* dstT = a.poolT ? reinterpret_cast<elem_t<DT>*>(a.poolT) + (((size_t)page * a.rank) << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1)) : nullptr;
+  const int row_w = a.rank + a.rot_dim;
+  elem_t<DT>* dst = reinterpret_cast<elem_t<DT>*>(a.pool) + (((size_t)page << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1))) * row_w;
+  elem_t<DT>* dstT = a.poolT ? reinterpret_cast<elem_t<DT>*>(a.poolT) + (((size_t)page * row_w) << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1)) : nullptr;
   for (int c = lane; c < a.rank; c += 64) {
     const elem_t<DT> v = f32_to_elem<DT>(s[c] * rinv * a.nw[c]);
     dst[c] = v;
     if (dstT) dstT[(size_t)c << m.page_shift] = v;
+  }
+  if (a.rot_dim <= 0) return;
+  const int half = a.rot_dims >> 1;
+  // vector 0 is the shared key part, vectors 1 .. heads the queries' rotated parts; element i of a vector: a rotated pair member or a channel that passes
+  for (int i = lane; i < (a.heads + 1) * a.rot_dim; i += 64) {
+    const int vec = i / a.rot_dim, ch = i - vec * a.rot_dim;
+    const float* src = vec == 0 ? s + a.rank : a.q + (size_t)t * a.lds + (size_t)(vec - 1) * a.qstride + a.qoff;
+    float v = src[ch];
+    if (ch < 2 * half) {
+      const int pr = ch < half ? ch : ch - half;
+      const float c = a.cs[((size_t)pos * half + pr) * 2], sn = a.cs[((size_t)pos * half + pr) * 2 + 1];
+      v = ch < half ? __fsub_rn(__fmul_rn(v, c), __fmul_rn(src[ch + half], sn)) : __fadd_rn(__fmul_rn(v, c), __fmul_rn(src[ch - half], sn));
+    }
+    if (vec == 0) {
+      const elem_t<DT> e = f32_to_elem<DT>(v);
+      dst[a.rank + ch] = e;
+      if (dstT) dstT[(size_t)(a.rank + ch) << m.page_shift] = e;
+    } else a.ql[(size_t)t * a.heads * row_w + (size_t)(vec - 1) * row_w + a.rank + ch] = v * a.qscale;
   }
 }
 
@@ -185,9 +211,10 @@ constexpr int LAT_MAX_RPL = 32;       // latent channels per lane: rank <= 2048
 struct LatentAttnArgs {
   const float* q; long long ldq;      // [T][heads * rank]
   const void* pool;
-  const float* sink;                  // [heads]
+  const float* sink;                  // [heads] (nullptr: the softmax has no sink)
   float* out; long long ldo;          // [T][heads * rank]
   int rank, heads;
+  int mask_kind, mask_size;           // MASK_*: the query at position i sees the keys [first_key(i), i] (stack_meta.h)
   // split form: keys [split * keys_per, ...) of every token's range; partial records (m, l, acc[rank]) per (token, head, split)
   float* part; int nsplit, keys_per;
 };
@@ -222,14 +249,14 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(StepMeta m, LatentAttn
   extern __shared__ float s_acc[];      // [4][rank]
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int row = m.tok_row[t], nkeys = m.tok_pos[t] + 1;
-  int k0 = 0, k1 = nkeys;
-  if (SPLIT) { k0 = min(nkeys, (int)blockIdx.z * a.keys_per); k1 = min(nkeys, k0 + a.keys_per); }
+  int k0 = first_key(nkeys - 1, a.mask_kind, a.mask_size), k1 = nkeys;
+  if (SPLIT) { k0 = min(nkeys, k0 + (int)blockIdx.z * a.keys_per); k1 = min(nkeys, k0 + a.keys_per); }
   const float* q = a.q + (size_t)t * a.ldq + (size_t)h * a.rank;
   float qv[RPL], acc[RPL];
 #pragma unroll
   for (int k = 0; k < RPL; k++) { const int c = lane + 64 * k; qv[k] = c < a.rank ? q[c] : 0.f; acc[k] = 0.f; }
   // the sink enters once: as the starting state of wave 0 (of split 0)
-  const bool has_sink = wv == 0 && (!SPLIT || blockIdx.z == 0);
+  const bool has_sink = a.sink && wv == 0 && (!SPLIT || blockIdx.z == 0);
   float mx = has_sink ? a.sink[h] : -INFINITY, l = has_sink ? 1.f : 0.f;
   latent_scan<DT, RPL>(m, a, row, k0 + wv, k1, 4, qv, mx, l, acc);
   if (lane == 0) { s_m[wv] = mx; s_l[wv] = l; }
@@ -245,7 +272,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(StepMeta m, LatentAttn
     if (threadIdx.x == 0) { rec[0] = M; rec[1] = L; }
     for (int c = threadIdx.x; c < a.rank; c += 256) rec[2 + c] = s_acc[c] * f[0] + s_acc[a.rank + c] * f[1] + s_acc[2 * a.rank + c] * f[2] + s_acc[3 * a.rank + c] * f[3];
   } else {
-    const float inv = 1.0f / L;
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
     float* o = a.out + (size_t)t * a.ldo + (size_t)h * a.rank;
     for (int c = threadIdx.x; c < a.rank; c += 256) o[c] = (s_acc[c] * f[0] + s_acc[a.rank + c] * f[1] + s_acc[2 * a.rank + c] * f[2] + s_acc[3 * a.rank + c] * f[3]) * inv;
   }
@@ -265,7 +292,7 @@ __global__ __launch_bounds__(256) void latent_attn_merge_kernel(LatentAttnArgs a
     float lf = s < a.nsplit ? rec[(size_t)s * rs + 1] * f : 0.f;
     for (int o = 1; o < 64; o <<= 1) { const float other = __shfl_up(lf, o, 64); if (s >= o) lf += other; }      // prefix sums: lane 63 holds the total in split order
     s_f[s] = f;
-    if (s == 63) s_inv = 1.0f / lf;
+    if (s == 63) s_inv = lf > 0.f ? 1.0f / lf : 0.f;
   }
   __syncthreads();
   const float inv = s_inv;

@@ -14,7 +14,7 @@
 
 namespace tgx {
 
-enum { SG_ACT_NONE = 0, SG_ACT_TANH = 1, SG_ACT_DECAY = 2 };
+enum { SG_ACT_NONE = 0, SG_ACT_TANH = 1, SG_ACT_DECAY = 2, SG_ACT_GELU = 3 };
 enum { SG_STORE = 0, SG_ADD = 1, SG_GATE = 2, SG_EXPERT_ACT = 3, SG_ROWSCALE = 4, SG_SILU_MUL = 5 };
 constexpr bool sg_dual(int epi) { return epi == SG_EXPERT_ACT || epi == SG_SILU_MUL; }
 struct StackGemmArgs {
@@ -26,12 +26,14 @@ struct StackGemmArgs {
   const int* z_off; const int* tile_z; const int* tile_m0; const int* n_tiles;      // grouped
   int M, N, K;
   float scale;                 // SG_STORE: C = act(acc * scale + bias); SG_ADD: C += acc * scale
-  int act;                     // SG_STORE: SG_ACT_NONE, SG_ACT_TANH, or SG_ACT_DECAY = exp(-exp(v)) (a decay in (0, 1) from a log-log pre-activation)
+  int act;                     // SG_STORE: SG_ACT_NONE, SG_ACT_TANH, SG_ACT_DECAY = exp(-exp(v)) (a decay in (0, 1) from a log-log pre-activation), or
+                               //           SG_ACT_GELU = v (1 + erf(v / sqrt 2)) / 2
   const float* bias;           // SG_STORE: [N] per z (column z * c_zoff + n), nullptr: none
   int gate_col0, gate_heads;   // SG_STORE: columns [gate_col0, + gate_heads) leave as log input gates cap tanh(v / cap), the next gate_heads columns as log forget gates
   float gate_cap;              //           logsigmoid(cap tanh(v / cap)) (the two gate rows of a matrix-memory layer's input product); gate_heads 0: none
   float limit;                 // SG_EXPERT_ACT
-  const float* G; long long ldg; int g_col0;     // SG_GATE: C = acc * sigmoid(G[row][g_col0 + z * c_zoff + n])
+  const float* G; long long ldg; int g_col0;     // SG_GATE: C = acc * sigmoid(G[row][g_col0 + z * c_zoff + n]), or with g_per_z
+  int g_per_z;                                   //          one gate per batch member z (a head): sigmoid(G[row][g_col0 + z])
   const float* rw;             // SG_ROWSCALE: C = acc * rw[c row]
   int terms;                   // 16-bit storage: 2 = hi + lo, 1 = hi only
 };
@@ -49,6 +51,7 @@ __device__ __forceinline__ float store_value(const StackGemmArgs& a, float v, si
   if (a.gate_heads > 0 && n >= a.gate_col0) { o = soft_cap(o, a.gate_cap); if (n >= a.gate_col0 + a.gate_heads) o = log_sigmoid(o); }
   if (a.act == SG_ACT_TANH) o = tanhf(o);
   else if (a.act == SG_ACT_DECAY) o = expf(-expf(o));
+  else if (a.act == SG_ACT_GELU) o = 0.5f * o * (1.0f + erff(o * 0.70710678118654752f));
   return o;
 }
 // the plain gated expert: silu(gate) * up
@@ -238,7 +241,7 @@ __global__ __launch_bounds__(256) void stack_gemm_kernel(const StackGemmArgs a) 
         const float v = acc[0][i][j][r];
         if constexpr (EPI == SG_STORE) cp[n] = store_value(a, v, (size_t)z * a.c_zoff + n, n);
         else if constexpr (EPI == SG_ADD) cp[n] = fmaf(v, a.scale, cp[n]);
-        else if constexpr (EPI == SG_GATE) cp[n] = v / (1.0f + expf(-a.G[crow * a.ldg + a.g_col0 + (size_t)z * a.c_zoff + n]));
+        else if constexpr (EPI == SG_GATE) cp[n] = v / (1.0f + expf(-a.G[crow * a.ldg + a.g_col0 + (a.g_per_z ? (size_t)z : (size_t)z * a.c_zoff + n)]));
         else if constexpr (EPI == SG_EXPERT_ACT) cp[n] = expert_act(v, acc[NB - 1][i][j][r], a.limit);
         else if constexpr (EPI == SG_SILU_MUL) cp[n] = silu_mul(v, acc[NB - 1][i][j][r]);
         else cp[n] = v * a.rw[crow];
@@ -336,7 +339,7 @@ __global__ __launch_bounds__(256) void stack_gemv_kernel(const StackGemmArgs a) 
       const float v = acc[0][j][r];
       if constexpr (EPI == SG_STORE) cp[n] = store_value(a, v, (size_t)z * a.c_zoff + n, n);
       else if constexpr (EPI == SG_ADD) cp[n] = fmaf(v, a.scale, cp[n]);
-      else if constexpr (EPI == SG_GATE) cp[n] = v / (1.0f + expf(-a.G[crow * a.ldg + a.g_col0 + (size_t)z * a.c_zoff + n]));
+      else if constexpr (EPI == SG_GATE) cp[n] = v / (1.0f + expf(-a.G[crow * a.ldg + a.g_col0 + (a.g_per_z ? (size_t)z : (size_t)z * a.c_zoff + n)]));
       else if constexpr (EPI == SG_EXPERT_ACT) cp[n] = expert_act(v, acc[NB - 1][j][r], a.limit);
       else if constexpr (EPI == SG_SILU_MUL) cp[n] = silu_mul(v, acc[NB - 1][j][r]);
       else cp[n] = v * a.rw[crow];

@@ -117,12 +117,25 @@ struct GqaAppendArgs {
   const float* lam;
   int rot_pairs;             // 1: neighbours turn together
   float q_temp_coef; int q_temp_every;      // coef 0: no query temperature
+  float qk_unit_eps;         // > 0: every q and k head is first divided by sqrt(mean(head^2) + qk_unit_eps) (no weight)
 };
 template <int DT>
 __global__ __launch_bounds__(256) void gqa_append_kernel(StepMeta m, GqaAppendArgs a) {
   const int t = blockIdx.x, pos = m.tok_pos[t];
   float* row = a.proj + (size_t)t * a.ldp;
   const int half = a.rot_dims >> 1, nh = a.heads + (a.poolK ? a.kv_heads : 0);      // q heads and k heads are adjacent in the row: head index hd, offset hd * dim
+  if (a.qk_unit_eps > 0.f) {      // a wave per head
+    const int lane = threadIdx.x & 63;
+    for (int hd = threadIdx.x >> 6; hd < nh; hd += 4) {
+      float* u = row + (size_t)hd * a.dim;
+      float ss = 0.f;
+      for (int c = lane; c < a.dim; c += 64) ss = fmaf(u[c], u[c], ss);
+      ss = wave_sum(ss);
+      const float r = 1.0f / sqrtf(ss / (float)a.dim + a.qk_unit_eps);
+      for (int c = lane; c < a.dim; c += 64) u[c] *= r;
+    }
+    __syncthreads();
+  }
   for (int i = threadIdx.x; i < nh * half; i += 256) {
     const int hd = i / half, p = i - hd * half;
     const float c = a.cs[((size_t)pos * half + p) * 2], s = a.cs[((size_t)pos * half + p) * 2 + 1];
@@ -425,6 +438,8 @@ __global__ __launch_bounds__(64) void head_norm_gate_kernel(HeadNormGateArgs a) 
 // there is one.  Scores s = softmax(z) over all E; choice scores c = s + corr; the E outputs form `groups` equal groups of neighbours, a group counts as
 // its largest choice score, members of the `keep` best groups stay eligible; the `top` largest eligible choice scores are chosen (ties: the lower index);
 // weights = s * scale.  One wave per token.
+// Variants: sigmoid_scores: s = sigmoid(z) instead of the softmax (corr may be nullptr: no correction); group_top2: a group counts as the sum of its two
+// largest choice scores; normalise: the chosen weights are divided by their sum + 1e-20 (before the scale).
 struct RouterGroupArgs {
   const float* z; int ldz;
   const float* corr;         // [E]
@@ -432,25 +447,30 @@ struct RouterGroupArgs {
   float* sgw;                // [T] sigmoid of the product in column E (nullptr: none)
   int E, top, groups, keep;
   float scale;
+  int sigmoid_scores, group_top2, normalise;
 };
 __global__ __launch_bounds__(64) void router_group_kernel(RouterGroupArgs a) {
   __shared__ float s_s[ROUTER_MAX_E], s_c[ROUTER_MAX_E], s_g[ROUTER_MAX_E];
   const int t = blockIdx.x, lane = threadIdx.x;
   const float* z = a.z + (size_t)t * a.ldz;
-  float mx = -INFINITY;
-  for (int e = lane; e < a.E; e += 64) mx = fmaxf(mx, z[e]);
-  mx = group_max<64>(mx);
-  float den = 0.f;
-  for (int e = lane; e < a.E; e += 64) { const float p = expf(z[e] - mx); s_s[e] = p; den += p; }
-  den = wave_sum(den);
-  for (int e = lane; e < a.E; e += 64) { s_s[e] = s_s[e] / den; s_c[e] = s_s[e] + a.corr[e]; }
+  if (a.sigmoid_scores) {
+    for (int e = lane; e < a.E; e += 64) { s_s[e] = 1.0f / (1.0f + expf(-z[e])); s_c[e] = a.corr ? s_s[e] + a.corr[e] : s_s[e]; }
+  } else {
+    float mx = -INFINITY;
+    for (int e = lane; e < a.E; e += 64) mx = fmaxf(mx, z[e]);
+    mx = group_max<64>(mx);
+    float den = 0.f;
+    for (int e = lane; e < a.E; e += 64) { const float p = expf(z[e] - mx); s_s[e] = p; den += p; }
+    den = wave_sum(den);
+    for (int e = lane; e < a.E; e += 64) { s_s[e] = s_s[e] / den; s_c[e] = a.corr ? s_s[e] + a.corr[e] : s_s[e]; }
+  }
   __syncthreads();
   if (a.groups > 1) {
     const int per = a.E / a.groups;
     for (int g = lane; g < a.groups; g += 64) {
-      float b = -INFINITY;
-      for (int e = g * per; e < (g + 1) * per; e++) b = fmaxf(b, s_c[e]);
-      s_g[g] = b;
+      float b = -INFINITY, b2 = -INFINITY;      // the largest and the second largest
+      for (int e = g * per; e < (g + 1) * per; e++) { const float v = s_c[e]; if (v > b) { b2 = b; b = v; } else b2 = fmaxf(b2, v); }
+      s_g[g] = a.group_top2 && per > 1 ? b + b2 : b;
     }
     __syncthreads();
     // the `keep` best groups, one pick per round; a kept group is marked by +inf, the others end as dropped
@@ -480,6 +500,12 @@ __global__ __launch_bounds__(64) void router_group_kernel(RouterGroupArgs a) {
       a.sel[(size_t)t * a.top + k] = pick;
       a.selw[(size_t)t * a.top + k] = bi < a.E ? s_s[pick] * a.scale : 0.f;
     }
+  }
+  if (a.normalise && lane == 0) {      // in choice order
+    float sum = 0.f;
+    for (int k = 0; k < a.top; k++) sum += a.selw[(size_t)t * a.top + k];
+    const float inv = a.scale / (sum + 1e-20f * a.scale);
+    for (int k = 0; k < a.top; k++) a.selw[(size_t)t * a.top + k] *= inv;
   }
   if (a.sgw && lane == 0) a.sgw[t] = 1.0f / (1.0f + expf(-z[a.E]));
 }

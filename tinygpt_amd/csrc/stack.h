@@ -47,6 +47,20 @@ struct StackLayerW {
   ebyte *w_o2 = nullptr, *w_w1 = nullptr, *w_w2 = nullptr;
   float *mu = nullptr, *w0 = nullptr, *ubonus = nullptr, *conv_w = nullptr, *a_log = nullptr, *dt_bias = nullptr;
   float* shift = nullptr;       // [2][slots][width]
+  // layer-norm designs (Zaluvik).  ln holds the layer's eight norm vectors [norm1 w | b | norm1b w | b | norm2 w | b | norm2b w | b][width].
+  //   attention:        w_in = [q | k | v | gate] rows (gate per output channel), talk the head-mixing matrix [heads][heads], pb the per-head score bias
+  //   latent attention: w_in = [q (heads * (dim + rot_dim)) | latent + rotated key part (kv_rank + rot_dim) | gate (heads)], w_ukT / w_uv / lat_norm as above
+  //   dense: w_up / w_down; experts: w_router (fp32), w_gate / w_up / w_down stacked, ws_* the shared expert
+  // The caches of these layers belong to their RUNS (StackModel::runs): a layer inside the loop has one per pass.
+  float *ln = nullptr, *talk = nullptr, *pb = nullptr;
+};
+
+// one run of a layer (layer-norm designs): which layer's weights, whether the loop's input product comes first, and the run's own cache
+struct StackRun {
+  int layer = 0;
+  bool inject = false;          // x <- W_loop [x; x0] in front of this run (the first layer of a pass of the loop)
+  ebyte* pool = nullptr;        // attention: keys [pages][page_tokens][kv_heads * dim]; latent attention: [pages][page_tokens][kv_rank + rot_dim]
+  ebyte* poolV = nullptr;       // attention: values [pages][page_tokens][kv_heads * vdim]
 };
 
 struct RotTable { int dims; float base; float factor; float* cs; };      // cos / sin of (position, pair) [max_ctx][dims / 2][2], angle = position * base^(-2 pair / dims) / factor, made on the host in double precision
@@ -59,6 +73,10 @@ struct StackModel {
   // what the family fixes (stack_create): the kind of norm and of layer wiring
   bool sandwich = false;               // scalar RMS norms before and after every sublayer, no convolutions, no depth average, no position vector, a separate head
   bool joint = false;                  // one offset-weight RMS norm per layer; mixer and feed-forward read it side by side; x += residual_mult * (their sum); a separate head
+  bool affine = false;                 // layer norms (weight and bias) before and after every sublayer, x += residual_mult * norm(sublayer(norm(x))); a looped span; logits against the embedding table
+  std::vector<StackRun> runs;          // affine designs: the layers in the order they run
+  ebyte* w_loop = nullptr;             // [width][2 width]: the loop's input product on [x; x0]
+  float* xcat = nullptr;               // step workspace [T][2 width]: the stream beside the embedding output
   float *mixed = nullptr, *lora = nullptr, *rec_in = nullptr;      // joint designs' step workspace: the token-shift mixes, the decay's inner product, the delta rule's inputs
   int max_shift = 0, max_lora = 0, max_rec = 0;
   ebyte* head = nullptr;               // [vocab][width] (sandwich and joint designs; the others multiply by the embedding table)

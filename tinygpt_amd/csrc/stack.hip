@@ -16,6 +16,7 @@
 #include "kernels/stack_seq.h"
 #include "kernels/stack_gqa_mfma.h"
 #include "kernels/stack_rec.h"
+#include "kernels/stack_loop.h"
 
 int upload_param_ext(tgx_ctx* c, ebyte* dst, const void* host, int64_t n, int src_dtype);      // abi.hip
 
@@ -171,7 +172,7 @@ int ensure_ws(tgx_ctx* c, int T) {
   auto fr = [](auto*& p) { if (p) (void)hipFree(p); p = nullptr; };
   fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw); fr(sm->yh); fr(sm->yd); fr(sm->xn); fr(sm->lg);
   fr(sm->sel); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->meta_dev); fr(sm->zr);
-  fr(sm->a2); fr(sm->ytmp); fr(sm->ysh); fr(sm->sgw); fr(sm->vfirst); fr(sm->hs); fr(sm->mixed); fr(sm->lora); fr(sm->rec_in);
+  fr(sm->a2); fr(sm->ytmp); fr(sm->ysh); fr(sm->sgw); fr(sm->vfirst); fr(sm->hs); fr(sm->mixed); fr(sm->lora); fr(sm->rec_in); fr(sm->xcat);
   if (sm->meta_host) { (void)hipHostFree(sm->meta_host); sm->meta_host = nullptr; }
   const int cap = std::max(T, 64);
   const size_t W = (size_t)sm->d.width, n = (size_t)cap;
@@ -179,6 +180,8 @@ int ensure_ws(tgx_ctx* c, int T) {
   if (sm->sandwich) {      // no layer results are kept; the seams need a second normed stream, a scratch row and the mixers' side buffers
     if ((rc = dev_alloc(c, &sm->a2, n * W)) || (rc = dev_alloc(c, &sm->ytmp, n * W)) || (rc = dev_alloc(c, &sm->ysh, n * W)) || (rc = dev_alloc(c, &sm->sgw, n)) ||
         (rc = dev_alloc(c, &sm->vfirst, n * (size_t)std::max(1, sm->max_kvv))) || (rc = dev_alloc(c, &sm->hs, n * (size_t)std::max(1, sm->max_hv)))) return rc;
+  } else if (sm->affine) {   // the seam's scratch row, the shared expert's row, the stream beside the embedding output
+    if ((rc = dev_alloc(c, &sm->ytmp, n * W)) || (rc = dev_alloc(c, &sm->ysh, n * W)) || (rc = dev_alloc(c, &sm->xcat, 2 * n * W))) return rc;
   } else if (sm->joint) {    // the recurrent mixers' side buffers: un-normed outputs, token-shift mixes, the decay's inner product, the delta rule's inputs
     if ((rc = dev_alloc(c, &sm->hs, n * (size_t)std::max(1, sm->max_hv))) || (rc = dev_alloc(c, &sm->mixed, n * (size_t)std::max(1, sm->max_shift))) ||
         (rc = dev_alloc(c, &sm->lora, n * (size_t)std::max(1, sm->max_lora))) || (rc = dev_alloc(c, &sm->rec_in, n * (size_t)std::max(1, sm->max_rec)))) return rc;
@@ -686,7 +689,407 @@ int run_layers_joint(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys,
   return TGX_OK;
 }
 
+// ---- layer-norm designs (Zaluvik): per run of a layer  x += mult * LN_b(mixer(LN_a(x)))  and  x += mult * LN_d(ff(LN_c(x))).  A run has its own cache (a layer
+// inside the loop runs once per pass); in front of the first layer of every pass the stream is replaced by the loop's input product on [x; x0].  The seam
+// kernel applies the norm behind a sublayer, the residual add and the norm in front of the next one.
+template <int DT, bool SPLIT>
+void launch_mix_attn_t(tgx_ctx* c, const tgx::StepMeta& m, const tgx::MixAttnArgs& a, dim3 grid, size_t lds, bool vec) {
+  const int npt = (a.heads * a.vdim + 255) / 256;
+  auto go = [&](auto N, auto V) {
+    constexpr int NPT = decltype(N)::value; constexpr bool VEC = decltype(V)::value;
+    auto* fn = &tgx::sigmoid_mix_attn_kernel<DT, NPT, VEC, SPLIT>;
+    if (lds > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(fn, grid, dim3(256), lds, c->stream, m, a);
+  };
+  auto gv = [&](auto N) { if (vec) go(N, std::true_type{}); else go(N, std::false_type{}); };
+  if (npt <= 1) gv(std::integral_constant<int, 1>{});
+  else if (npt <= 2) gv(std::integral_constant<int, 2>{});
+  else if (npt <= 4) gv(std::integral_constant<int, 4>{});
+  else if (npt <= 8) gv(std::integral_constant<int, 8>{});
+  else if (npt <= 16) gv(std::integral_constant<int, 16>{});
+  else gv(std::integral_constant<int, 32>{});
+}
+constexpr int MIX_ATTN_MAX_OUT = 32 * 256;            // heads * vdim of the sigmoid attention (output channels per thread <= 32)
+constexpr size_t MIX_ATTN_MAX_LDS = 144 * 1024;
+int mix_attn_tile_keys(int heads, int dim) {          // keys per tile: as many as keep the workgroup's LDS within 64 KB, 64 at least
+  for (int kt = 256; kt > 64; kt >>= 1) if (tgx::mix_attn_lds_bytes(heads, dim, kt) <= 64 * 1024) return kt;
+  return 64;
+}
+
+int run_affine_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const StackRun& run, int T, int max_keys) {
+  StackModel* sm = c->stack;
+  const tgx_layer_desc& ld = w.d;
+  const int W = sm->d.width, H = ld.heads, G = ld.kv_heads, qd = H * ld.dim, kd = G * ld.dim, kvv = G * ld.vdim, vd = H * ld.vdim, nin = qd + kd + kvv + vd;
+  // [q | k | v | gate] = h . w_in^T
+  tgx::StackGemmArgs g{};
+  g.A = sm->a; g.lda = W; g.B = w.w_in; g.ldb = W; g.C = sm->proj; g.ldc = nin; g.M = T; g.N = nin; g.K = W; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  tgx::GqaAppendArgs ap{};
+  ap.proj = sm->proj; ap.ldp = nin; ap.heads = H; ap.kv_heads = G; ap.dim = ld.dim; ap.vdim = ld.vdim; ap.poolK = run.pool; ap.poolV = run.poolV;
+  ap.qk_unit_eps = ld.qk_norm ? sm->d.norm_eps : 0.f;
+  TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::gqa_append_kernel<DT>, dim3(T), dim3(256), 0, c->stream, m, ap))
+  tgx::MixAttnArgs aa{};
+  aa.q = sm->proj; aa.ldq = nin; aa.poolK = run.pool; aa.poolV = run.poolV; aa.pb = w.pb; aa.talk = ld.head_mix ? w.talk : nullptr;
+  aa.gate = ld.gate_kind == 1 ? sm->proj + qd + kd + kvv : nullptr; aa.ldg = nin; aa.out = sm->o; aa.ldo = vd;
+  aa.heads = H; aa.kv_heads = G; aa.dim = ld.dim; aa.vdim = ld.vdim; aa.scale = ld.scale; aa.mask_kind = ld.mask_kind; aa.mask_size = ld.mask_size;
+  aa.kt = mix_attn_tile_keys(H, ld.dim);
+  const size_t lds = tgx::mix_attn_lds_bytes(H, ld.dim, aa.kt);
+  const bool vec = ld.dim % 8 == 0;
+  const int span = ld.mask_kind == tgx::MASK_CAUSAL ? max_keys : std::min(max_keys, ld.mask_size);
+  int nsplit = 1;
+  if (span >= sm->gqa_split_min_keys && (long long)T < c->num_cus) {      // few tokens and a long span: the keys are divided between workgroups, whole tiles each
+    nsplit = (int)std::min<long long>(64, (2LL * c->num_cus) / T);
+    const int per = std::max(aa.kt, ((span + nsplit - 1) / nsplit + aa.kt - 1) / aa.kt * aa.kt);
+    nsplit = (span + per - 1) / per;
+    aa.keys_per = per;
+  }
+  if (nsplit > 1) {
+    int rc = ensure_part(c, (size_t)T * nsplit * (size_t)vd);
+    if (rc) return rc;
+    aa.part = sm->part; aa.nsplit = nsplit;
+    TGX_DT_SWITCH(c->dt, (launch_mix_attn_t<DT, true>(c, m, aa, dim3(T, nsplit), lds, vec)))
+    hipLaunchKernelGGL(tgx::sigmoid_mix_merge_kernel, dim3(T, std::min(8, (vd + 255) / 256)), dim3(256), 0, c->stream, aa);
+  } else {
+    TGX_DT_SWITCH(c->dt, (launch_mix_attn_t<DT, false>(c, m, aa, dim3(T), lds, vec)))
+  }
+  // y = o . w_o^T
+  g = tgx::StackGemmArgs{};
+  g.A = sm->o; g.lda = vd; g.B = w.w_o; g.ldb = vd; g.C = sm->yd; g.ldc = W; g.M = T; g.N = W; g.K = vd; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  return TGX_OK;
+}
+
+// latent attention with a rotated key part that all heads share and a window: the pool row is [normed latent | rotated key part]; every head's query is
+// taken into that space ([scale W_uk^T q_plain | scale rot(q_rot)]), so a score is one dot product with the cached row and nothing else is cached
+int run_affine_latent(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const StackRun& run, int T, int max_keys) {
+  StackModel* sm = c->stack;
+  const tgx_layer_desc& ld = w.d;
+  const int W = sm->d.width, H = ld.heads, qs = ld.dim + ld.rot_dim, qd = H * qs, R = ld.kv_rank, RR = R + ld.rot_dim, vd = H * ld.vdim, ng = ld.gate_kind == 2 ? H : vd, nin = qd + RR + ng;
+  tgx::StackGemmArgs g{};
+  g.A = sm->a; g.lda = W; g.B = w.w_in; g.ldb = W; g.C = sm->proj; g.ldc = nin; g.M = T; g.N = nin; g.K = W; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  tgx::LatentAppendArgs la{};
+  la.src = sm->proj; la.lds = nin; la.col0 = qd; la.nw = w.lat_norm; la.pool = run.pool; la.rank = R; la.eps = sm->d.norm_eps;
+  la.rot_dim = ld.rot_dim; la.rot_dims = ld.rot_dims; la.cs = w.rot >= 0 ? sm->rot[(size_t)w.rot].cs : nullptr;
+  la.q = sm->proj; la.heads = H; la.qstride = qs; la.qoff = ld.dim; la.qscale = ld.scale; la.ql = sm->ql;
+  TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::latent_append_kernel<DT>, dim3(T), dim3(64), 0, c->stream, m, la))
+  // the plain part of every head's query into latent space: ql[t][h][0 .. R) = scale * q_plain[t][h] . ukT[h]^T
+  g = tgx::StackGemmArgs{};
+  g.A = sm->proj; g.lda = nin; g.a_zoff = qs; g.B = w.w_ukT; g.ldb = ld.dim; g.b_zstride = (long long)R * ld.dim; g.C = sm->ql; g.ldc = (long long)H * RR; g.c_zoff = RR;
+  g.M = T; g.N = R; g.K = ld.dim; g.scale = ld.scale;
+  launch_gemm(c, g, tgx::SG_STORE, H);
+  tgx::LatentAttnArgs aa{};
+  aa.q = sm->ql; aa.ldq = (long long)H * RR; aa.pool = run.pool; aa.sink = nullptr; aa.out = sm->lat; aa.ldo = (long long)H * RR; aa.rank = RR; aa.heads = H;
+  aa.mask_kind = ld.mask_kind; aa.mask_size = ld.mask_size;
+  const int span = ld.mask_kind == tgx::MASK_CAUSAL ? max_keys : std::min(max_keys, ld.mask_size);
+  int nsplit = 1;
+  if (span >= sm->attn_split_min_keys && (long long)T * H < 2LL * c->num_cus) {
+    nsplit = (int)std::min<long long>(64, (4LL * c->num_cus) / ((long long)T * H));
+    const int per = std::max(256, ((span + nsplit - 1) / nsplit + 63) / 64 * 64);
+    nsplit = (span + per - 1) / per;
+    aa.keys_per = per;
+  }
+  if (nsplit > 1) {
+    int rc = ensure_part(c, (size_t)T * H * nsplit * (size_t)(RR + 2));
+    if (rc) return rc;
+    aa.part = sm->part; aa.nsplit = nsplit;
+    TGX_DT_SWITCH(c->dt, (launch_attn_t<DT, true>(c, m, aa, dim3(T, H, nsplit))))
+    hipLaunchKernelGGL(tgx::latent_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, aa);
+  } else {
+    TGX_DT_SWITCH(c->dt, (launch_attn_t<DT, false>(c, m, aa, dim3(T, H))))
+  }
+  // o[t][h] = (lat[t][h][0 .. R) . uv[h]^T) * sigmoid(gate of the head, or of the channel)
+  g = tgx::StackGemmArgs{};
+  g.A = sm->lat; g.lda = (long long)H * RR; g.a_zoff = RR; g.B = w.w_uv; g.ldb = R; g.b_zstride = (long long)ld.vdim * R; g.C = sm->o; g.ldc = vd; g.c_zoff = ld.vdim;
+  g.M = T; g.N = ld.vdim; g.K = R; g.G = sm->proj; g.ldg = nin; g.g_col0 = qd + RR; g.g_per_z = ld.gate_kind == 2;
+  launch_gemm(c, g, tgx::SG_GATE, H);
+  g = tgx::StackGemmArgs{};
+  g.A = sm->o; g.lda = vd; g.B = w.w_o; g.ldb = vd; g.C = sm->yd; g.ldc = W; g.M = T; g.N = W; g.K = vd; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 1);
+  return TGX_OK;
+}
+
+// the feed-forward of a layer-norm design into yd (one row per token, or `top` rows per token for experts) and ysh (the shared expert's row)
+void run_affine_ff(tgx_ctx* c, StackLayerW& w, int T) {
+  StackModel* sm = c->stack;
+  const tgx_layer_desc& ld = w.d;
+  const int W = sm->d.width;
+  tgx::StackGemmArgs g{};
+  if (ld.mlp == TGX_MLP_DENSE) {      // down(act(up h))
+    g.A = sm->a; g.lda = W; g.B = w.w_up; g.ldb = W; g.C = sm->yh; g.ldc = ld.ff; g.M = T; g.N = ld.ff; g.K = W; g.scale = 1.f; g.act = ld.ff_act == 1 ? tgx::SG_ACT_GELU : tgx::SG_ACT_NONE;
+    launch_gemm(c, g, tgx::SG_STORE, 1);
+    g = tgx::StackGemmArgs{};
+    g.A = sm->yh; g.lda = ld.ff; g.B = w.w_down; g.ldb = ld.ff; g.C = sm->yd; g.ldc = W; g.M = T; g.N = W; g.K = ld.ff; g.scale = 1.f;
+    launch_gemm(c, g, tgx::SG_STORE, 1);
+    return;
+  }
+  const int E = ld.experts, top = ld.top, np = T * top;
+  g.A = sm->a; g.lda = W; g.B = w.w_router; g.ldb = W; g.C = sm->zr; g.ldc = E; g.M = T; g.N = E; g.K = W; g.scale = 1.f;
+  launch_gemm(c, g, tgx::SG_STORE, 1, 0, 0, 64, tgx::DT_F32);
+  tgx::RouterGroupArgs ra{};
+  ra.z = sm->zr; ra.ldz = E; ra.corr = nullptr; ra.sel = sm->sel; ra.selw = sm->selw; ra.sgw = nullptr;
+  ra.E = E; ra.top = top; ra.groups = ld.groups; ra.keep = ld.groups_keep; ra.scale = 1.f;
+  ra.sigmoid_scores = ld.router_fn == 1; ra.group_top2 = ld.group_score == 1; ra.normalise = ld.router_norm;
+  hipLaunchKernelGGL(tgx::router_group_kernel, dim3(T), dim3(64), 0, c->stream, ra);
+  tgx::MoePlanArgs pa{};
+  pa.sel = sm->sel; pa.n_pairs = np; pa.E = E; pa.top = top; pa.tile_m = grouped_tile_rows(c, np, W, ld.ff); pa.E_tiles = E;
+  pa.off = sm->moe_off; pa.perm = sm->perm; pa.tok = sm->ptok; pa.tile_e = sm->tile_e; pa.tile_m0 = sm->tile_m0; pa.n_tiles = sm->n_tiles;
+  hipLaunchKernelGGL(tgx::moe_plan_kernel, dim3(1), dim3(1024), 0, c->stream, pa);
+  g = tgx::StackGemmArgs{};
+  g.A = sm->a; g.lda = W; g.a_rows = sm->ptok; g.B = w.w_gate; g.B2 = w.w_up; g.ldb = W; g.b_zstride = (long long)ld.ff * W; g.C = sm->yh; g.ldc = ld.ff;
+  g.z_off = sm->moe_off; g.tile_z = sm->tile_e; g.tile_m0 = sm->tile_m0; g.n_tiles = sm->n_tiles; g.M = np; g.N = ld.ff; g.K = W;
+  launch_gemm(c, g, tgx::SG_SILU_MUL, 1, np, E, pa.tile_m);
+  g = tgx::StackGemmArgs{};
+  g.A = sm->yh; g.lda = ld.ff; g.B = w.w_down; g.ldb = ld.ff; g.b_zstride = (long long)W * ld.ff; g.C = sm->yd; g.ldc = W; g.c_rows = sm->perm;
+  g.z_off = sm->moe_off; g.tile_z = sm->tile_e; g.tile_m0 = sm->tile_m0; g.n_tiles = sm->n_tiles; g.M = np; g.N = W; g.K = ld.ff; g.rw = sm->selw;
+  launch_gemm(c, g, tgx::SG_ROWSCALE, 1, np, E, pa.tile_m);
+  if (ld.shared_ff > 0) {      // the shared expert runs for every token, without a gate of its own
+    float* hsh = sm->yh + (size_t)np * std::max(1, ld.ff);
+    g = tgx::StackGemmArgs{};
+    g.A = sm->a; g.lda = W; g.B = w.ws_gate; g.B2 = w.ws_up; g.ldb = W; g.C = hsh; g.ldc = ld.shared_ff; g.M = T; g.N = ld.shared_ff; g.K = W;
+    launch_gemm(c, g, tgx::SG_SILU_MUL, 1);
+    g = tgx::StackGemmArgs{};
+    g.A = hsh; g.lda = ld.shared_ff; g.B = w.ws_down; g.ldb = ld.shared_ff; g.C = sm->ysh; g.ldc = W; g.M = T; g.N = W; g.K = ld.shared_ff; g.scale = 1.f;
+    launch_gemm(c, g, tgx::SG_STORE, 1);
+  }
+}
+
+int run_layers_affine(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys) {
+  StackModel* sm = c->stack;
+  const tgx::StepMeta m = step_meta(sm, mp, T, S);
+  const int W = sm->d.width;
+  const float eps = sm->d.norm_eps, mult = sm->d.residual_mult;
+  const bool looped = sm->w_loop != nullptr;
+  TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::embed_scale_rows_kernel<DT>, dim3(T), dim3(256), 0, c->stream, m, reinterpret_cast<const tgx::elem_t<DT>*>(c->embed), sm->d.embed_scale,
+                                          sm->x, looped ? sm->xcat + W : nullptr, 2LL * W, W))
+  bool normed = false;      // whether sm->a holds the next sublayer's normed input
+  for (size_t ri = 0; ri < sm->runs.size(); ri++) {
+    const StackRun& run = sm->runs[ri];
+    StackLayerW& w = sm->L[(size_t)run.layer];
+    const tgx_layer_desc& ld = w.d;
+    const float* ln = w.ln;
+    if (run.inject) {      // x <- W_loop [x; x0]
+      hipLaunchKernelGGL(tgx::copy_rows_kernel, dim3(T), dim3(256), 0, c->stream, sm->x, (long long)W, sm->xcat, 2LL * W, W);
+      tgx::StackGemmArgs g{};
+      g.A = sm->xcat; g.lda = 2LL * W; g.B = sm->w_loop; g.ldb = 2LL * W; g.C = sm->x; g.ldc = W; g.M = T; g.N = W; g.K = 2 * W; g.scale = 1.f;
+      launch_gemm(c, g, tgx::SG_STORE, 1);
+      normed = false;
+    }
+    if (!normed) hipLaunchKernelGGL(tgx::layer_norm_rows_kernel, dim3(T), dim3(256), 0, c->stream, sm->x, nullptr, ln, ln + W, sm->a, W, eps);
+    int rc = ld.mixer == TGX_MIXER_ATTENTION ? run_affine_attention(c, m, w, run, T, max_keys) : run_affine_latent(c, m, w, run, T, max_keys);
+    if (rc) return rc;
+    const bool last = ri + 1 == sm->runs.size();
+    const bool next_direct = !last && !sm->runs[ri + 1].inject;      // the next run's first norm can ride in this run's last seam
+    const float* next_ln = next_direct ? sm->L[(size_t)sm->runs[ri + 1].layer].ln : nullptr;
+    tgx::AffineSeamArgs sa{};
+    sa.x = sm->x; sa.y = sm->yd; sa.top = 1; sa.ytmp = sm->ytmp; sa.w_post = ln + 2 * (size_t)W; sa.b_post = ln + 3 * (size_t)W; sa.mult = mult; sa.out = sm->a; sa.W = W; sa.eps = eps;
+    if (ld.mlp != TGX_MLP_NONE) { sa.w_next = ln + 4 * (size_t)W; sa.b_next = ln + 5 * (size_t)W; }
+    else if (next_ln) { sa.w_next = next_ln; sa.b_next = next_ln + W; }
+    hipLaunchKernelGGL(tgx::affine_seam_kernel, dim3(T), dim3(256), 0, c->stream, sa);
+    normed = sa.w_next != nullptr;
+    if (ld.mlp == TGX_MLP_NONE) continue;
+    run_affine_ff(c, w, T);
+    sa = tgx::AffineSeamArgs{};
+    sa.x = sm->x; sa.y = sm->yd; sa.top = ld.mlp == TGX_MLP_MOE ? ld.top : 1; sa.ysh = ld.mlp == TGX_MLP_MOE && ld.shared_ff > 0 ? sm->ysh : nullptr; sa.ytmp = sm->ytmp;
+    sa.w_post = ln + 6 * (size_t)W; sa.b_post = ln + 7 * (size_t)W; sa.mult = mult; sa.out = sm->a; sa.W = W; sa.eps = eps;
+    if (next_ln) { sa.w_next = next_ln; sa.b_next = next_ln + W; }
+    hipLaunchKernelGGL(tgx::affine_seam_kernel, dim3(T), dim3(256), 0, c->stream, sa);
+    normed = sa.w_next != nullptr;
+  }
+  return TGX_OK;
+}
+
+// parameter storage of a layer-norm design (Zaluvik) and the list of its layer runs
+int create_affine_layers(tgx_ctx* c, const tgx_layer_desc* layers) {
+  StackModel* sm = c->stack;
+  const tgx_stack_desc& d = sm->d;
+  const size_t W = (size_t)d.width, es = c->esz;
+  int rc;
+  auto need = [&](const std::string& p, std::initializer_list<const char*> names) { for (const char* n : names) sm->missing.insert(p + n); };
+  sm->missing.insert("final.norm.b");
+  const bool looped = d.loop_times > 1 && d.loop_stop > d.loop_start;
+  if (looped) {
+    if ((rc = dev_alloc(c, &sm->w_loop, W * 2 * W * es))) return rc;
+    sm->missing.insert("loop.in");
+  }
+  for (int i = 0; i < d.layers; i++) {
+    const int reps = looped && i >= d.loop_start && i < d.loop_stop ? 1 : 0;
+    if (looped && i == d.loop_start) {
+      for (int t = 0; t < d.loop_times; t++)
+        for (int j = d.loop_start; j < d.loop_stop; j++) { StackRun r; r.layer = j; r.inject = j == d.loop_start; sm->runs.push_back(r); }
+    }
+    if (!reps) { StackRun r; r.layer = i; sm->runs.push_back(r); }
+  }
+  sm->max_top = 1; sm->max_E = 1; sm->max_ff = 1;      // the mixers' outputs and the dense feed-forward use the expert buffers with one row per token
+  for (int i = 0; i < d.layers; i++) {
+    StackLayerW& w = sm->L[(size_t)i];
+    w.d = layers[i];
+    const tgx_layer_desc& l = w.d;
+    const std::string p = "l" + std::to_string(i) + ".";
+    const size_t H = (size_t)l.heads, vd = H * l.vdim;
+    if ((rc = dev_alloc(c, &w.ln, 8 * W))) return rc;
+    HIP_OK(c, hipMemset(w.ln, 0, 8 * W * 4));
+    need(p, {"norm1", "norm1.b", "norm1b", "norm1b.b", "mix.q", "mix.g", "mix.o"});
+    size_t nin;
+    if (l.mixer == TGX_MIXER_ATTENTION) {
+      const size_t qd = H * l.dim, kd = (size_t)l.kv_heads * l.dim, kvv = (size_t)l.kv_heads * l.vdim;
+      nin = qd + kd + kvv + vd;
+      if ((rc = dev_alloc(c, &w.talk, H * H)) || (rc = dev_alloc(c, &w.pb, H))) return rc;
+      HIP_OK(c, hipMemset(w.pb, 0, H * 4));
+      need(p, {"mix.k", "mix.v"});
+      if (l.head_mix) need(p, {"mix.talk"});
+      if (l.score_fn == 1) need(p, {"mix.pb"});
+    } else {
+      const size_t qd = H * (size_t)(l.dim + l.rot_dim), R = (size_t)l.kv_rank, RR = R + l.rot_dim;
+      nin = qd + RR + (l.gate_kind == 2 ? H : vd);
+      if ((rc = dev_alloc(c, &w.w_ukT, H * l.dim * R * es)) || (rc = dev_alloc(c, &w.w_uv, vd * R * es)) || (rc = dev_alloc(c, &w.lat_norm, R))) return rc;
+      need(p, {"mix.dkv", "mix.dkv.norm", "mix.uk", "mix.uv"});
+      if (l.rot_dim > 0 && l.rot_dims > 0) {
+        for (size_t r = 0; r < sm->rot.size(); r++) if (sm->rot[r].dims == l.rot_dims && sm->rot[r].base == l.rot_base) w.rot = (int)r;
+        if (w.rot < 0) { w.rot = (int)sm->rot.size(); sm->rot.push_back(RotTable{l.rot_dims, l.rot_base, 1.f, nullptr}); }
+      }
+      sm->max_hr = std::max(sm->max_hr, (int)(H * RR));
+    }
+    if ((rc = dev_alloc(c, &w.w_in, nin * W * es)) || (rc = dev_alloc(c, &w.w_o, W * vd * es))) return rc;
+    sm->max_in = std::max(sm->max_in, (int)nin); sm->max_hv = std::max(sm->max_hv, (int)vd);
+    if (l.mlp == TGX_MLP_NONE) continue;
+    need(p, {"norm2", "norm2.b", "norm2b", "norm2b.b"});
+    if (l.mlp == TGX_MLP_DENSE) {
+      const size_t F = (size_t)l.ff;
+      if ((rc = dev_alloc(c, &w.w_up, F * W * es)) || (rc = dev_alloc(c, &w.w_down, W * F * es))) return rc;
+      need(p, {"mlp.up", "mlp.down"});
+      sm->max_ff = std::max(sm->max_ff, l.ff);
+      continue;
+    }
+    const size_t E = (size_t)l.experts, F = (size_t)l.ff, SF = (size_t)l.shared_ff;
+    if ((rc = dev_alloc(c, &w.w_router, E * W)) || (rc = dev_alloc(c, &w.w_gate, E * F * W * es)) || (rc = dev_alloc(c, &w.w_up, E * F * W * es)) || (rc = dev_alloc(c, &w.w_down, E * W * F * es))) return rc;
+    need(p, {"mlp.router"});
+    for (int e = 0; e < l.experts; e++)
+      for (const char* n : {".gate", ".up", ".down"}) sm->missing.insert(p + "mlp.e" + std::to_string(e) + n);
+    if (SF > 0) {
+      if ((rc = dev_alloc(c, &w.ws_gate, SF * W * es)) || (rc = dev_alloc(c, &w.ws_up, SF * W * es)) || (rc = dev_alloc(c, &w.ws_down, W * SF * es))) return rc;
+      need(p, {"mlp.shared.gate", "mlp.shared.up", "mlp.shared.down"});
+    }
+    sm->max_top = std::max(sm->max_top, l.top); sm->max_ff = std::max(sm->max_ff, l.ff); sm->max_E = std::max(sm->max_E, l.experts); sm->max_sff = std::max(sm->max_sff, l.shared_ff);
+  }
+  return TGX_OK;
+}
+
+// tensors of a layer-norm design by checkpoint name; a norm is a weight vector and a bias vector ("<name>.b")
+int upload_affine(tgx_ctx* c, const char* name, const void* host, const int64_t* shape, int nd, int src_dtype) {
+  StackModel* sm = c->stack;
+  const tgx_stack_desc& d = sm->d;
+  const int64_t W = d.width;
+  const bool probe = nd < 0;
+  auto bad_shape = [&]() { return set_err(c, TGX_ERR_SHAPE, "shape not equal for tensor: %s", name); };
+  auto is = [&](int64_t a, int64_t b) { return b < 0 ? (nd == 1 && shape[0] == a) : (nd == 2 && shape[0] == a && shape[1] == b); };
+  auto done = [&](int rc) { if (!rc) sm->missing.erase(name); return rc; };
+  auto mat = [&](ebyte* dst, int64_t row0, int64_t rows, int64_t cols) {
+    if (probe) return (int)TGX_ERR_SHAPE;
+    if (!is(rows, cols)) return bad_shape();
+    return done(upload_param_ext(c, dst + (size_t)(row0 * cols) * c->esz, host, rows * cols, src_dtype));
+  };
+  auto vec = [&](float* dst, int64_t n, int64_t n2 = -1) {      // an fp32 vector, or (n2 >= 0) an fp32 matrix [n][n2]
+    if (probe) return (int)TGX_ERR_SHAPE;
+    if (!is(n, n2)) return bad_shape();
+    return done(upload_f32(c, dst, host, n2 < 0 ? n : n * n2, src_dtype));
+  };
+  if (!strcmp(name, "embed")) return mat(c->embed, 0, d.vocab, W);
+  if (!strcmp(name, "final.norm")) return vec(sm->final_norm, W);
+  if (!strcmp(name, "final.norm.b")) return vec(sm->final_norm + W, W);
+  if (sm->w_loop && !strcmp(name, "loop.in")) return mat(sm->w_loop, 0, W, 2 * W);
+  int li = -1;
+  char rest[128] = {0};
+  if (sscanf(name, "l%d.%127s", &li, rest) != 2 || li < 0 || li >= d.layers) return set_err(c, TGX_ERR_NAME, "Unexpected key: %s", name);
+  StackLayerW& w = sm->L[(size_t)li];
+  const tgx_layer_desc& l = w.d;
+  const int64_t H = l.heads, vd = H * l.vdim;
+  static const char* const norms[8] = {"norm1", "norm1.b", "norm1b", "norm1b.b", "norm2", "norm2.b", "norm2b", "norm2b.b"};
+  for (int k = 0; k < (l.mlp == TGX_MLP_NONE ? 4 : 8); k++) if (!strcmp(rest, norms[k])) return vec(w.ln + (size_t)k * W, W);
+  if (!strcmp(rest, "mix.o")) return mat(w.w_o, 0, W, vd);
+  if (l.mixer == TGX_MIXER_ATTENTION) {
+    const int64_t qd = H * l.dim, kd = (int64_t)l.kv_heads * l.dim, kvv = (int64_t)l.kv_heads * l.vdim;
+    if (!strcmp(rest, "mix.q")) return mat(w.w_in, 0, qd, W);
+    if (!strcmp(rest, "mix.k")) return mat(w.w_in, qd, kd, W);
+    if (!strcmp(rest, "mix.v")) return mat(w.w_in, qd + kd, kvv, W);
+    if (!strcmp(rest, "mix.g")) return mat(w.w_in, qd + kd + kvv, vd, W);
+    if (l.head_mix && !strcmp(rest, "mix.talk")) return vec(w.talk, H, H);
+    if (l.score_fn == 1 && !strcmp(rest, "mix.pb")) return vec(w.pb, H);
+  } else {
+    const int64_t qd = H * (int64_t)(l.dim + l.rot_dim), R = l.kv_rank, RR = R + l.rot_dim;
+    if (!strcmp(rest, "mix.q")) return mat(w.w_in, 0, qd, W);
+    if (!strcmp(rest, "mix.dkv")) return mat(w.w_in, qd, RR, W);
+    if (!strcmp(rest, "mix.g")) return mat(w.w_in, qd + RR, l.gate_kind == 2 ? H : vd, W);
+    if (!strcmp(rest, "mix.dkv.norm")) return vec(w.lat_norm, R);
+    if (!strcmp(rest, "mix.uv")) return mat(w.w_uv, 0, vd, R);
+    if (!strcmp(rest, "mix.uk")) {      // [heads * dim][rank] -> per head [rank][dim]
+      if (probe) return TGX_ERR_SHAPE;
+      if (!is(H * l.dim, R)) return bad_shape();
+      const size_t es = esize(src_dtype);
+      std::vector<unsigned char> t((size_t)(H * l.dim * R) * es);
+      const unsigned char* src = (const unsigned char*)host;
+      for (int64_t h = 0; h < H; h++)
+        for (int64_t dd = 0; dd < l.dim; dd++)
+          for (int64_t r = 0; r < R; r++) memcpy(&t[(size_t)((h * R + r) * l.dim + dd) * es], src + (size_t)((h * l.dim + dd) * R + r) * es, es);
+      return done(upload_param_ext(c, w.w_ukT, t.data(), H * l.dim * R, src_dtype));
+    }
+  }
+  if (l.mlp == TGX_MLP_DENSE) {
+    if (!strcmp(rest, "mlp.up")) return mat(w.w_up, 0, l.ff, W);
+    if (!strcmp(rest, "mlp.down")) return mat(w.w_down, 0, W, l.ff);
+  }
+  if (l.mlp == TGX_MLP_MOE) {
+    const int64_t E = l.experts, F = l.ff, SF = l.shared_ff;
+    if (!strcmp(rest, "mlp.router")) return vec(w.w_router, E, W);
+    if (SF > 0) {
+      if (!strcmp(rest, "mlp.shared.gate")) return mat(w.ws_gate, 0, SF, W);
+      if (!strcmp(rest, "mlp.shared.up")) return mat(w.ws_up, 0, SF, W);
+      if (!strcmp(rest, "mlp.shared.down")) return mat(w.ws_down, 0, W, SF);
+    }
+    int e = -1;
+    char leaf[32] = {0};
+    if (sscanf(rest, "mlp.e%d.%31s", &e, leaf) == 2 && e >= 0 && e < E) {
+      if (!strcmp(leaf, "gate")) return mat(w.w_gate, e * F, F, W);
+      if (!strcmp(leaf, "up")) return mat(w.w_up, e * F, F, W);
+      if (!strcmp(leaf, "down")) return mat(w.w_down, e * W, W, F);
+    }
+  }
+  return set_err(c, TGX_ERR_NAME, "Unexpected key: %s", name);
+}
+
+// what a layer-norm design's description may ask for
+int check_affine_desc(const tgx_stack_desc& d, const tgx_layer_desc* layers) {
+  if (d.loop_times > 1 && d.loop_stop > d.loop_start && (d.loop_start < 0 || d.loop_stop > d.layers)) return set_err(nullptr, TGX_ERR_INVALID, "loop %d .. %d outside the %d layers", d.loop_start, d.loop_stop, d.layers);
+  for (int i = 0; i < d.layers; i++) {
+    const tgx_layer_desc& l = layers[i];
+    if (l.heads <= 0 || l.dim <= 0 || l.vdim <= 0) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: non-positive mixer size", i);
+    if (l.mask_kind < 0 || l.mask_kind > 2 || (l.mask_kind != 0 && l.mask_size < 1)) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: mask", i);
+    if (l.mixer == TGX_MIXER_ATTENTION) {
+      if (l.kv_heads <= 0 || l.heads % l.kv_heads) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: %d query heads over %d key / value heads", i, l.heads, l.kv_heads);
+      if (l.score_fn != 1) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: this family's attention takes sigmoid weights (score_fn 1)", i);
+      if ((long long)l.heads * l.vdim > MIX_ATTN_MAX_OUT || tgx::mix_attn_lds_bytes(l.heads, l.dim, 64) > MIX_ATTN_MAX_LDS)
+        return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: sigmoid attention: %d heads of %d / %d exceed the kernel's %d output channels or its LDS", i, l.heads, l.dim, l.vdim, MIX_ATTN_MAX_OUT);
+      if (l.gate_kind != 0 && l.gate_kind != 1) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: attention gates are per channel", i);
+    } else if (l.mixer == TGX_MIXER_LATENT_ATTENTION) {
+      if (l.kv_rank <= 0 || l.rot_dim < 0 || l.kv_rank + l.rot_dim > 64 * tgx::LAT_MAX_RPL) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: kv_rank %d + rot_dim %d (1 .. %d)", i, l.kv_rank, l.rot_dim, 64 * tgx::LAT_MAX_RPL);
+      if (l.rot_dim > 0 && (l.rot_dims < 0 || l.rot_dims > l.rot_dim || (l.rot_dims & 1) || (l.rot_dims > 0 && !(l.rot_base > 0.f)))) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: %d rotated dimensions of %d (base %g)", i, l.rot_dims, l.rot_dim, l.rot_base);
+      if (l.gate_kind != 1 && l.gate_kind != 2) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: latent attention gates are per channel or per head", i);
+    } else return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: mixer %d is not part of this family (attention and latent_attention are)", i, l.mixer);
+    if (l.mlp != TGX_MLP_NONE && l.mlp != TGX_MLP_MOE && l.mlp != TGX_MLP_DENSE) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: feed-forward kind %d is not implemented", i, l.mlp);
+    if (l.mlp == TGX_MLP_DENSE && l.ff <= 0) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: ff %d", i, l.ff);
+    if (l.mlp == TGX_MLP_MOE) {
+      const int E = l.experts;
+      if (E <= 0 || E >= tgx::ROUTER_MAX_E || l.top <= 0 || l.top > E || l.top > tgx::ROUTER_MAX_TOP || l.ff <= 0 || l.shared_ff < 0 || l.identity != 0)
+        return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: experts %d (< %d), top %d (<= %d), ff %d", i, E, tgx::ROUTER_MAX_E, l.top, tgx::ROUTER_MAX_TOP, l.ff);
+      if (l.groups > 1 && (E % l.groups || l.groups_keep < 1 || l.groups_keep > l.groups || (long long)l.groups_keep * (E / l.groups) < l.top))
+        return set_err(nullptr, TGX_ERR_INVALID, "layer %d: %d experts in %d groups, %d kept, top %d", i, E, l.groups, l.groups_keep, l.top);
+    }
+  }
+  return TGX_OK;
+}
+
 int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int max_count) {
+  if (c->stack->affine) return run_layers_affine(c, mp, T, S, max_keys);
   if (c->stack->joint) return run_layers_joint(c, mp, T, S, max_keys, max_count);
   return c->stack->sandwich ? run_layers_sandwich(c, mp, T, S, max_keys, max_count) : run_layers_latent(c, mp, T, S, max_keys, max_count);
 }
@@ -695,7 +1098,8 @@ int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int m
 void run_logits(tgx_ctx* c, const int* want_dev, int nw, float* C, const int* c_rows) {
   StackModel* sm = c->stack;
   const int W = sm->d.width, V = sm->d.vocab;
-  if (sm->joint) hipLaunchKernelGGL(tgx::offset_norm_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->final_norm, 1.0f, sm->xn, W, sm->d.norm_eps);
+  if (sm->affine) hipLaunchKernelGGL(tgx::layer_norm_rows_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->final_norm, sm->final_norm + W, sm->xn, W, sm->d.norm_eps);
+  else if (sm->joint) hipLaunchKernelGGL(tgx::offset_norm_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->final_norm, 1.0f, sm->xn, W, sm->d.norm_eps);
   else if (sm->sandwich) hipLaunchKernelGGL(tgx::scalar_norm_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->norm_g + 4 * (size_t)sm->d.layers, sm->xn, W, sm->d.norm_eps);
   else hipLaunchKernelGGL(tgx::final_norm_rows_kernel, dim3(nw), dim3(256), 0, c->stream, sm->x, want_dev, sm->final_norm, sm->xn, W, sm->d.norm_groups, sm->d.norm_eps);
   tgx::StackGemmArgs g{};
@@ -1054,16 +1458,17 @@ int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int d
   if (!desc || !layers || !out_ctx) return set_err(nullptr, TGX_ERR_INVALID, "null argument");
   *out_ctx = nullptr;
   const tgx_stack_desc& d = *desc;
-  if (d.family != TGX_FAMILY_ZAKUSUN && d.family != TGX_FAMILY_MODEPEL && d.family != TGX_FAMILY_VITUDRA) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "family %d is not a layered model", d.family);
-  const bool sandwich = d.family == TGX_FAMILY_MODEPEL, joint = d.family == TGX_FAMILY_VITUDRA;
+  if (d.family != TGX_FAMILY_ZAKUSUN && d.family != TGX_FAMILY_MODEPEL && d.family != TGX_FAMILY_VITUDRA && d.family != TGX_FAMILY_ZALUVIK) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "family %d is not a layered model", d.family);
+  const bool sandwich = d.family == TGX_FAMILY_MODEPEL, joint = d.family == TGX_FAMILY_VITUDRA, affine = d.family == TGX_FAMILY_ZALUVIK;
   if (d.width <= 0 || d.layers <= 0 || d.vocab <= 0 || d.max_seqs <= 0 || d.max_ctx <= 0) return set_err(nullptr, TGX_ERR_INVALID, "non-positive model dimension");
   if (d.compute_dtype != TGX_BF16 && d.compute_dtype != TGX_F16 && d.compute_dtype != TGX_F32) return set_err(nullptr, TGX_ERR_INVALID, "unknown compute dtype %d", d.compute_dtype);
-  if (!sandwich && !joint && (d.norm_groups < 1 || d.norm_groups > tgx::NORM_MAX_GROUPS || d.width % d.norm_groups)) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "norm groups %d: 1..%d, dividing the width", d.norm_groups, tgx::NORM_MAX_GROUPS);
-  if (!sandwich && !joint && (d.canon_taps < 1 || d.canon_taps > tgx::CONV_MAX_TAPS)) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "convolution taps %d: 1..%d", d.canon_taps, tgx::CONV_MAX_TAPS);
+  if (affine) { const int rc = check_affine_desc(d, layers); if (rc) return rc; }
+  if (!sandwich && !joint && !affine && (d.norm_groups < 1 || d.norm_groups > tgx::NORM_MAX_GROUPS || d.width % d.norm_groups)) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "norm groups %d: 1..%d, dividing the width", d.norm_groups, tgx::NORM_MAX_GROUPS);
+  if (!sandwich && !joint && !affine && (d.canon_taps < 1 || d.canon_taps > tgx::CONV_MAX_TAPS)) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "convolution taps %d: 1..%d", d.canon_taps, tgx::CONV_MAX_TAPS);
   int page = d.page_tokens > 0 ? d.page_tokens : 64;
   if (page & (page - 1)) return set_err(nullptr, TGX_ERR_INVALID, "page_tokens %d is not a power of two", page);
   int first_mix = -1;
-  for (int i = 0; i < d.layers; i++) {
+  for (int i = 0; i < d.layers && !affine; i++) {
     const tgx_layer_desc& l = layers[i];
     if (joint) {
       auto attention_ok = [&](const char*& why) {
@@ -1141,8 +1546,8 @@ int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int d
   while ((1 << sm->page_shift) < page) sm->page_shift++;
   // what the shared sampler / token rings read from the flat description
   c->d.family = d.family; c->d.hidden = d.width; c->d.layers = d.layers; c->d.vocab = d.vocab; c->d.max_ctx = d.max_ctx; c->d.max_batch = d.max_seqs;
-  c->d.compute_dtype = d.compute_dtype; c->d.tied = sandwich || joint ? 0 : 1; c->d.norm_eps = d.norm_eps;
-  sm->sandwich = sandwich; sm->joint = joint;
+  c->d.compute_dtype = d.compute_dtype; c->d.tied = sandwich || joint ? 0 : 1; c->d.norm_eps = d.norm_eps;      // (a layer-norm design multiplies by the embedding table)
+  sm->sandwich = sandwich; sm->joint = joint; sm->affine = affine;
   c->device = device_ordinal;
   c->dt = d.compute_dtype == TGX_BF16 ? tgx::DT_BF16 : (d.compute_dtype == TGX_F16 ? tgx::DT_F16 : tgx::DT_F32);
   c->esz = d.compute_dtype == TGX_F32 ? 4 : 2;
@@ -1154,11 +1559,12 @@ int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int d
 
   const size_t W = (size_t)d.width, es = c->esz;
   int rc;
-  if ((rc = dev_alloc(c, &c->embed, (size_t)d.vocab * W * es)) || (rc = dev_alloc(c, &sm->final_norm, W))) return rc;
+  if ((rc = dev_alloc(c, &c->embed, (size_t)d.vocab * W * es)) || (rc = dev_alloc(c, &sm->final_norm, 2 * W))) return rc;      // (weight, and a bias where the norm has one)
   sm->missing.insert("embed"); sm->missing.insert("final.norm");
   sm->L.resize((size_t)d.layers);
   if (sandwich) return create_sandwich_layers(c, layers);
   if (joint) return create_joint_layers(c, layers);
+  if (affine) return create_affine_layers(c, layers);
   for (int i = 0; i < d.layers; i++) {
     StackLayerW& w = sm->L[(size_t)i];
     w.d = layers[i];
@@ -1199,6 +1605,7 @@ int stack_upload(tgx_ctx* c, const char* name, const void* host, const int64_t* 
   if (src_dtype != TGX_BF16 && src_dtype != TGX_F32 && src_dtype != TGX_F16) return set_err(c, TGX_ERR_INVALID, "unknown source dtype %d", src_dtype);
   if (sm->sandwich) return upload_sandwich(c, name, host, shape, nd, src_dtype);
   if (sm->joint) return upload_joint(c, name, host, shape, nd, src_dtype);
+  if (sm->affine) return upload_affine(c, name, host, shape, nd, src_dtype);
   if (!strcmp(name, "embed")) { if (probe) return TGX_ERR_SHAPE; if (!is(d.vocab, W)) return bad_shape(); return done(upload_param_ext(c, c->embed, host, d.vocab * W, src_dtype)); }
   if (!strcmp(name, "final.norm")) { if (probe) return TGX_ERR_SHAPE; if (!is(W, -1)) return bad_shape(); return done(upload_f32(c, sm->final_norm, host, W, src_dtype)); }
   int li = -1;
@@ -1262,7 +1669,7 @@ int stack_finalize(tgx_ctx* c) {
   const size_t W = (size_t)d.width, B = (size_t)d.max_seqs, V = (size_t)d.vocab;
   int rc;
   // angles of the position vector: pos * base^(-2i / width), the factor rounded to fp32 once
-  if (!sm->sandwich && !sm->joint) {
+  if (!sm->sandwich && !sm->joint && !sm->affine) {
     std::vector<float> fq(W / 2 + 1);
     for (size_t i = 0; i < fq.size(); i++) fq[i] = (float)pow(10000.0, -2.0 * (double)i / (double)W);
     if ((rc = dev_alloc(c, &sm->freq, fq.size()))) return rc;
@@ -1278,7 +1685,7 @@ int stack_finalize(tgx_ctx* c) {
   memset(sm->tbl_host, 0, B * (size_t)sm->tbl_stride * 4);
   sm->row_pages.assign(B, 0); sm->row_par.assign(B, 0); sm->row_dirty.assign(B, 0);
   for (int p = sm->n_pages - 1; p >= 0; p--) sm->free_pages.push_back(p);
-  const size_t nb = sm->sandwich || sm->joint ? 0 : (size_t)d.canon_taps - 1;
+  const size_t nb = sm->sandwich || sm->joint || sm->affine ? 0 : (size_t)d.canon_taps - 1;
   for (auto& r : sm->rot) {      // angle of (position, pair i) = position * base^(-2i / dims), evaluated in double, stored as fp32 cosine and sine
     const size_t half = (size_t)r.dims / 2;
     std::vector<float> cs((size_t)d.max_ctx * half * 2);
@@ -1289,7 +1696,22 @@ int stack_finalize(tgx_ctx* c) {
     if ((rc = dev_alloc(c, &r.cs, cs.size()))) return rc;
     HIP_OK(c, hipMemcpy(r.cs, cs.data(), cs.size() * 4, hipMemcpyHostToDevice));
   }
+  for (auto& run : sm->runs) {      // layer-norm designs: every run of a layer has its own cache
+    const tgx_layer_desc& l = sm->L[(size_t)run.layer].d;
+    const size_t rows = (size_t)sm->n_pages * sm->page;
+    if (l.mixer == TGX_MIXER_ATTENTION) {
+      const size_t ke = rows * (size_t)l.kv_heads * l.dim * c->esz, ve = rows * (size_t)l.kv_heads * l.vdim * c->esz;
+      if ((rc = dev_alloc(c, &run.pool, ke)) || (rc = dev_alloc(c, &run.poolV, ve))) return rc;
+      HIP_OK(c, hipMemset(run.pool, 0, ke));
+      HIP_OK(c, hipMemset(run.poolV, 0, ve));
+    } else {
+      const size_t pe = rows * (size_t)(l.kv_rank + l.rot_dim) * c->esz;
+      if ((rc = dev_alloc(c, &run.pool, pe))) return rc;
+      HIP_OK(c, hipMemset(run.pool, 0, pe));
+    }
+  }
   for (auto& w : sm->L) {
+    if (sm->affine) break;
     if (sm->joint) {
       const tgx_layer_desc& l = w.d;
       if (l.mixer != TGX_MIXER_WKV && w.kv_src < 0) {      // keys and values of an attention layer / a parallel mixer's attention half (a sharing layer borrows below)
@@ -1408,6 +1830,9 @@ void stack_destroy(tgx_ctx* c) {
     fr(w.b_in); fr(w.poolV); fr(w.poolVT); fr(w.vmix); fr(w.head_w); fr(w.mS); fr(w.mn); fr(w.mm); fr(w.act); fr(w.ws_gate); fr(w.ws_up); fr(w.ws_down);
   }
   for (auto& r : sm->rot) fr(r.cs);
+  for (auto& r : sm->runs) { fr(r.pool); fr(r.poolV); }
+  for (auto& w : sm->L) { fr(w.ln); fr(w.talk); fr(w.pb); }
+  fr(sm->w_loop); fr(sm->xcat);
   fr(sm->mixed); fr(sm->lora); fr(sm->rec_in);
   fr(sm->head); fr(sm->norm_g); fr(sm->a2); fr(sm->ytmp); fr(sm->ysh); fr(sm->sgw); fr(sm->vfirst); fr(sm->hs);
   fr(sm->final_norm); fr(sm->freq); fr(sm->tbl_dev); fr(sm->meta_dev); fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw);
@@ -1569,11 +1994,16 @@ int stack_read_latent(tgx_ctx* c, int row, int layer, float* out) {
   HIP_OK(c, hipStreamSynchronize(c->stream));
   const StackLayerW& w = sm->L[(size_t)layer];
   if ((sm->sandwich && w.d.mixer != TGX_MIXER_ATTENTION) || (sm->joint && !w.pool)) return set_err(c, TGX_ERR_UNSUPPORTED, "read_kv: layer %d caches no rows (its state is recurrent)", layer);
-  const size_t R = sm->sandwich || sm->joint ? (size_t)w.d.kv_heads * w.d.dim : (size_t)w.d.kv_rank;      // an attention layer's cached keys, all key heads of a token in a row
+  const ebyte* pool = w.pool;
+  size_t R = sm->sandwich || sm->joint ? (size_t)w.d.kv_heads * w.d.dim : (size_t)w.d.kv_rank;      // an attention layer's cached keys, all key heads of a token in a row
+  if (sm->affine) {      // the cache of the layer's first run: an attention layer's keys, a latent layer's rows [latent | rotated key part]
+    for (const StackRun& r : sm->runs) if (r.layer == layer) { pool = r.pool; break; }
+    R = w.d.mixer == TGX_MIXER_ATTENTION ? (size_t)w.d.kv_heads * w.d.dim : (size_t)(w.d.kv_rank + w.d.rot_dim);
+  }
   std::vector<unsigned char> buf(R * c->esz);
   for (int64_t t = 0; t < c->row_past[(size_t)row]; t++) {
     const size_t page = (size_t)sm->tbl_host[(size_t)row * sm->tbl_stride + (size_t)(t >> sm->page_shift)];
-    HIP_OK(c, hipMemcpy(buf.data(), w.pool + ((page << sm->page_shift) + (size_t)(t & (sm->page - 1))) * R * c->esz, R * c->esz, hipMemcpyDeviceToHost));
+    HIP_OK(c, hipMemcpy(buf.data(), pool + ((page << sm->page_shift) + (size_t)(t & (sm->page - 1))) * R * c->esz, R * c->esz, hipMemcpyDeviceToHost));
     const std::vector<float> f = to_f32(buf.data(), (int64_t)R, c->d.compute_dtype);
     memcpy(out + (size_t)t * R, f.data(), R * 4);
   }
@@ -1586,6 +2016,18 @@ int64_t stack_bytes_per_token(const tgx_ctx* c, int64_t T) {
   const int64_t W = sm->d.width, es = (int64_t)c->esz;
   int64_t b = (int64_t)sm->d.vocab * W * es;
   if (sm->sandwich || sm->joint) b *= 2;      // embedding row aside, the head is a matrix of its own
+  if (sm->affine) {      // per run of a layer: its matrices (the chosen experts only) and the rows of its cache inside the mask's span
+    if (sm->w_loop) b += (int64_t)sm->d.loop_times * 2 * W * W * es;
+    for (const StackRun& r : sm->runs) {
+      const tgx_layer_desc& l = sm->L[(size_t)r.layer].d;
+      const int64_t H = l.heads, vd = H * l.vdim, keys = l.mask_kind ? std::min<int64_t>(T, l.mask_size) : T;
+      if (l.mixer == TGX_MIXER_ATTENTION) b += ((H * l.dim + (int64_t)l.kv_heads * (l.dim + l.vdim) + vd) * W + W * vd) * es + keys * l.kv_heads * (l.dim + l.vdim) * es;
+      else b += ((H * (l.dim + l.rot_dim) + l.kv_rank + l.rot_dim + H) * W + (H * l.dim + vd) * l.kv_rank + W * vd) * es + keys * (l.kv_rank + l.rot_dim) * es;
+      if (l.mlp == TGX_MLP_DENSE) b += 2 * (int64_t)l.ff * W * es;
+      if (l.mlp == TGX_MLP_MOE) b += (int64_t)l.experts * W * 4 + (int64_t)l.top * 3 * l.ff * W * es + (int64_t)3 * l.shared_ff * W * es;
+    }
+    return b;
+  }
   for (const auto& w : sm->L) {
     const tgx_layer_desc& l = w.d;
     const int64_t H = l.heads, qd = H * l.dim, R = l.kv_rank, vd = H * l.vdim;

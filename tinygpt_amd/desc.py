@@ -271,12 +271,14 @@ def known_desc(key: str, compute_dtype: str | None = None, max_batch: int = 1) -
 FAMILY_ZAKUSUN = 6
 FAMILY_MODEPEL = 7
 FAMILY_VITUDRA = 8
-STACK_FAMILY = {"zakusun": FAMILY_ZAKUSUN, "modepel": FAMILY_MODEPEL, "vitudra": FAMILY_VITUDRA}
+FAMILY_ZALUVIK = 9
+STACK_FAMILY = {"zakusun": FAMILY_ZAKUSUN, "modepel": FAMILY_MODEPEL, "vitudra": FAMILY_VITUDRA, "zaluvik": FAMILY_ZALUVIK}
 MIXER_BY_NAME = {"latent_attention": 1, "attention": 2, "mlstm": 3, "wkv": 4, "parallel": 5}
 MLP_BY_NAME = {None: 0, "moe": 1, "dense": 2}
 MASK_BY_NAME = {None: 0, "window": 1, "chunk": 2}
 # which mixers a design is made of (config.json "architecture" -> layer "type")
-MIXERS_OF = {"zakusun": ("latent_attention",), "modepel": ("attention", "mlstm"), "vitudra": ("attention", "wkv", "parallel")}
+MIXERS_OF = {"zakusun": ("latent_attention",), "modepel": ("attention", "mlstm"), "vitudra": ("attention", "wkv", "parallel"),
+             "zaluvik": ("attention", "latent_attention")}
 
 
 class CLayerDesc(ctypes.Structure):
@@ -291,7 +293,10 @@ class CLayerDesc(ctypes.Structure):
                 ("q_temp_coef", ctypes.c_float), ("q_temp_every", ctypes.c_int32), ("rot_pairs", ctypes.c_int32), ("rot_factor", ctypes.c_float),
                 ("kv_share", ctypes.c_int32), ("decay_rank", ctypes.c_int32), ("d_heads", ctypes.c_int32), ("d_kv_heads", ctypes.c_int32),
                 ("d_dim", ctypes.c_int32), ("d_vdim", ctypes.c_int32), ("conv_taps", ctypes.c_int32), ("left_scale", ctypes.c_float),
-                ("right_scale", ctypes.c_float)]
+                ("right_scale", ctypes.c_float),
+                ("qk_norm", ctypes.c_int32), ("score_fn", ctypes.c_int32), ("head_mix", ctypes.c_int32), ("gate_kind", ctypes.c_int32),
+                ("rot_dim", ctypes.c_int32), ("ff_act", ctypes.c_int32), ("router_fn", ctypes.c_int32), ("group_score", ctypes.c_int32),
+                ("router_norm", ctypes.c_int32)]
 
 
 class CStackDesc(ctypes.Structure):
@@ -299,7 +304,8 @@ class CStackDesc(ctypes.Structure):
     _fields_ = [("family", ctypes.c_int32), ("width", ctypes.c_int32), ("layers", ctypes.c_int32), ("vocab", ctypes.c_int32),
                 ("compute_dtype", ctypes.c_int32), ("max_seqs", ctypes.c_int32), ("max_ctx", ctypes.c_int32),
                 ("budget_tokens", ctypes.c_int32), ("page_tokens", ctypes.c_int32), ("norm_groups", ctypes.c_int32),
-                ("norm_eps", ctypes.c_float), ("canon_taps", ctypes.c_int32), ("logit_scale", ctypes.c_float), ("residual_mult", ctypes.c_float)]
+                ("norm_eps", ctypes.c_float), ("canon_taps", ctypes.c_int32), ("logit_scale", ctypes.c_float), ("residual_mult", ctypes.c_float),
+                ("embed_scale", ctypes.c_float), ("loop_start", ctypes.c_int32), ("loop_stop", ctypes.c_int32), ("loop_times", ctypes.c_int32)]
 
 
 @dataclass
@@ -348,6 +354,17 @@ class LayerDesc:
     conv_taps: int = 0
     left_scale: float = 1.0
     right_scale: float = 1.0
+    # the layer-norm design (Zaluvik): unit queries and keys, sigmoid weights mixed across heads, the kind of output gate, the rotated part of a
+    # latent layer's queries and keys, the dense feed-forward's activation, the sigmoid router
+    qk_norm: bool = False
+    score_fn: "str | None" = None     # None: softmax; "sigmoid": sigmoid(score + per-head bias), not normalised over the keys
+    head_mix: bool = False
+    gate_kind: "str | None" = None    # None: the family's own; "channel" | "head"
+    rot_dim: int = 0
+    ff_act: "str | None" = None       # None: the family's own; "gelu"
+    router_fn: "str | None" = None    # None: softmax + correction; "sigmoid"
+    group_score: "str | None" = None  # None: a group's largest score; "top2": the sum of its two largest
+    router_norm: bool = False
 
     def to_c(self) -> CLayerDesc:
         return CLayerDesc(MIXER_BY_NAME[self.mixer], self.heads, self.dim, self.vdim, self.kv_rank, self.scale,
@@ -356,7 +373,10 @@ class LayerDesc:
                           self.groups_keep, self.router_scale, self.shared_ff,
                           MASK_BY_NAME[self.mask], self.mask_size, self.softcap, int(self.dist_bias), self.q_temp_coef, self.q_temp_every,
                           int(self.rot_pairs), self.rot_factor, 0 if self.kv_from is None else self.kv_from + 1, self.decay_rank,
-                          self.d_heads, self.d_kv_heads, self.d_dim, self.d_vdim, self.conv_taps, self.left_scale, self.right_scale)
+                          self.d_heads, self.d_kv_heads, self.d_dim, self.d_vdim, self.conv_taps, self.left_scale, self.right_scale,
+                          int(self.qk_norm), {None: 0, "sigmoid": 1}[self.score_fn], int(self.head_mix), {None: 0, "channel": 1, "head": 2}[self.gate_kind],
+                          self.rot_dim, {None: 0, "gelu": 1}[self.ff_act], {None: 0, "sigmoid": 1}[self.router_fn], {None: 0, "top2": 1}[self.group_score],
+                          int(self.router_norm))
 
 
 @dataclass
@@ -375,7 +395,11 @@ class StackDesc:
     norm_eps: float = 1e-6
     canon_taps: int = 1
     logit_scale: float = 1.0
-    residual_mult: float = 1.0   # Vitudra: the factor on what a layer adds to the stream
+    residual_mult: float = 1.0   # Vitudra, Zaluvik: the factor on what a (sub)layer adds to the stream
+    embed_scale: float = 1.0     # Zaluvik: the factor on the embedding rows
+    loop_start: int = 0          # Zaluvik: layers loop_start .. loop_stop - 1 run loop_times times with the same weights, a cache per pass
+    loop_stop: int = 0
+    loop_times: int = 1
     name: str = ""
 
     # the fields the flat description shares (bench / reporting code reads them)
@@ -389,8 +413,20 @@ class StackDesc:
         arr = (CLayerDesc * len(self.layers))(*[l.to_c() for l in self.layers])
         sd = CStackDesc(STACK_FAMILY[self.family], self.width, len(self.layers), self.vocab, DTYPE_BY_NAME[self.compute_dtype], self.max_seqs,
                         self.max_ctx, self.budget_tokens, self.page_tokens, self.norm_groups, self.norm_eps, self.canon_taps,
-                        self.logit_scale, self.residual_mult)
+                        self.logit_scale, self.residual_mult, self.embed_scale, self.loop_start, self.loop_stop, self.loop_times)
         return sd, arr
+
+    @property
+    def looped(self) -> bool:
+        return self.loop_times > 1 and self.loop_stop > self.loop_start
+
+    def layer_runs(self) -> "list[int]":
+        """the layers in the order they run (a looped span repeats)"""
+        n = len(self.layers)
+        if not self.looped:
+            return list(range(n))
+        span = list(range(self.loop_start, self.loop_stop))
+        return list(range(self.loop_start)) + span * self.loop_times + list(range(self.loop_stop, n))
 
     def tensor_shapes(self) -> "dict[str, tuple]":
         """checkpoint name -> shape, in file order"""
@@ -400,6 +436,8 @@ class StackDesc:
             return self._modepel_shapes(out)
         if self.family == "vitudra":
             return _vitudra_shapes(self, out)
+        if self.family == "zaluvik":
+            return _zaluvik_shapes(self, out)
         for i, l in enumerate(self.layers):
             p = f"l{i}."
             out[p + "norm1"] = (W,)
@@ -488,6 +526,66 @@ def _vitudra_shapes(self: StackDesc, out: dict) -> dict:
 
 
 
+def _zaluvik_shapes(self: StackDesc, out: dict) -> dict:
+    """checkpoint names and shapes of a Zaluvik model, in file order"""
+    W = self.width
+    if self.looped:
+        out["loop.in"] = (W, 2 * W)
+    for i, l in enumerate(self.layers):
+        p = f"l{i}."
+        for n in ("norm1", "norm2", "norm1b", "norm2b") if l.mlp else ("norm1", "norm1b"):
+            out[p + n] = (W,); out[p + n + ".b"] = (W,)
+        if l.mixer == "attention":
+            out[p + "mix.q"] = (l.heads * l.dim, W); out[p + "mix.k"] = (l.kv_heads * l.dim, W); out[p + "mix.v"] = (l.kv_heads * l.vdim, W)
+            out[p + "mix.talk"] = (l.heads, l.heads); out[p + "mix.pb"] = (l.heads,)
+            out[p + "mix.g"] = (l.heads * l.vdim, W); out[p + "mix.o"] = (W, l.heads * l.vdim)
+        else:
+            out[p + "mix.q"] = (l.heads * (l.dim + l.rot_dim), W); out[p + "mix.dkv"] = (l.kv_rank + l.rot_dim, W); out[p + "mix.dkv.norm"] = (l.kv_rank,)
+            out[p + "mix.uk"] = (l.heads * l.dim, l.kv_rank); out[p + "mix.uv"] = (l.heads * l.vdim, l.kv_rank)
+            out[p + "mix.g"] = (l.heads, W); out[p + "mix.o"] = (W, l.heads * l.vdim)
+        if l.mlp == "dense":
+            out[p + "mlp.up"] = (l.ff, W); out[p + "mlp.down"] = (W, l.ff)
+        elif l.mlp == "moe":
+            for e in range(l.experts):
+                out[p + f"mlp.e{e}.gate"] = (l.ff, W); out[p + f"mlp.e{e}.up"] = (l.ff, W); out[p + f"mlp.e{e}.down"] = (W, l.ff)
+            out[p + "mlp.router"] = (l.experts, W)
+            if l.shared_ff:
+                out[p + "mlp.shared.gate"] = (l.shared_ff, W); out[p + "mlp.shared.up"] = (l.shared_ff, W); out[p + "mlp.shared.down"] = (W, l.shared_ff)
+    out["final.norm"] = (W,); out["final.norm.b"] = (W,)
+    return out
+
+
+def _zaluvik_layer(i: int, l: dict) -> LayerDesc:
+    """one entry of a Zaluvik config's "layers": {"type": "attention" | "latent_attention", "mixer": {...}, "mlp": null | {"kind": "dense" | "moe", ...}}.
+    Attention: unit queries and keys, a sliding window, sigmoid weights with a per-head bias mixed across heads, a gate per output channel.
+    Latent attention: `rot_dim` rotated dimensions beside `dim` per head, one rotated key part for all heads, a sliding window, softmax, a gate per head."""
+    m, f = l["mixer"], l.get("mlp")
+    ld = LayerDesc(mixer=l["type"], heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]))
+    if m.get("mask"):
+        ld.mask = "window"; ld.mask_size = int(m["mask"]["size"])
+    if l["type"] == "attention":
+        ld.kv_heads = int(m.get("kv_heads", m["heads"])); ld.qk_norm = True; ld.score_fn = "sigmoid"; ld.head_mix = True; ld.gate_kind = "channel"
+    else:
+        rot = m.get("rot") or {}
+        ld.kv_rank = int(m["kv_rank"]); ld.rot_dim = int(m.get("rot_dim", 0)); ld.gate_kind = "head"
+        ld.rot_dims = int(rot.get("dims", ld.rot_dim)) if ld.rot_dim else 0; ld.rot_base = float(rot.get("base", 10000.0))
+        if ld.rot_dims > ld.rot_dim:
+            raise ValueError(f"layer {i}: {ld.rot_dims} rotated dimensions of a rotated part of {ld.rot_dim}")
+    if f is None:
+        return ld
+    if f.get("kind") == "dense":
+        ld.mlp = "dense"; ld.ff = int(f["ff"]); ld.ff_act = "gelu"
+    elif f.get("kind") == "moe":
+        r, g = f["router"], f["router"].get("groups") or {}
+        ld.mlp = "moe"; ld.experts = int(r["experts"]); ld.top = int(r["top"]); ld.ff = int(f["expert"]["ff"])
+        ld.groups = int(g.get("count", 1)); ld.groups_keep = int(g.get("keep", ld.groups))
+        ld.router_fn = "sigmoid"; ld.group_score = "top2"; ld.router_norm = True
+        ld.shared_ff = int(f["shared"]["ff"]) if f.get("shared") else 0
+    else:
+        raise ValueError(f"layer {i}: feed-forward kind {f.get('kind')!r} is not implemented")
+    return ld
+
+
 def _attention_fields(ld: LayerDesc, m: dict, mask: str):
     """the attention entries of a Vitudra mixer (an "attention" layer's, or the "left" half of a "parallel" one); what is absent is off"""
     ld.heads = int(m["heads"]); ld.kv_heads = int(m.get("kv_heads", m["heads"])); ld.dim = int(m["dim"]); ld.vdim = int(m.get("vdim", m["dim"]))
@@ -553,7 +651,7 @@ def _modepel_layer(i: int, l: dict) -> LayerDesc:
 
 
 def stack_desc_from_config(cfg: dict, compute_dtype: str = "bf16", max_seqs: int = 4, max_ctx: int = 4096, budget_tokens: int = 0, tensor_shapes=None) -> StackDesc:
-    """config.json of a layered model ("architecture": "Zakusun" | "Modepel" | "Vitudra") -> StackDesc.  Every size and constant comes from the file;
+    """config.json of a layered model ("architecture": "Zakusun" | "Modepel" | "Vitudra" | "Zaluvik") -> StackDesc.  Every size and constant comes from the file;
     tensor_shapes (checkpoint name -> shape, optional) gives the sizes that only a tensor's shape tells (a wkv layer's decay rank; left open without it:
     the device library then takes it from the tensor at upload)."""
     arch = str(cfg.get("architecture")).lower()
@@ -568,6 +666,13 @@ def stack_desc_from_config(cfg: dict, compute_dtype: str = "bf16", max_seqs: int
         return StackDesc(family="vitudra", width=int(cfg["width"]), vocab=int(cfg["vocab"]), layers=layers, compute_dtype=compute_dtype, max_seqs=max_seqs,
                          max_ctx=max_ctx, budget_tokens=budget_tokens, norm_groups=1, norm_eps=float(cfg["norm"]["eps"]), canon_taps=1, logit_scale=1.0,
                          residual_mult=float(cfg.get("residual_mult", 1.0)), name="vitudra")
+    if arch == "zaluvik":
+        lp = cfg.get("loop") or {}
+        return StackDesc(family="zaluvik", width=int(cfg["width"]), vocab=int(cfg["vocab"]), layers=[_zaluvik_layer(i, l) for i, l in enumerate(cfg["layers"])],
+                         compute_dtype=compute_dtype, max_seqs=max_seqs, max_ctx=max_ctx, budget_tokens=budget_tokens, norm_groups=1,
+                         norm_eps=float(cfg["norm"]["eps"]), canon_taps=1, logit_scale=1.0, residual_mult=float(cfg.get("residual_mult", 1.0)),
+                         embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)), loop_start=int(lp.get("start", 0)), loop_stop=int(lp.get("stop", 0)),
+                         loop_times=int(lp.get("times", 1)), name="zaluvik")
     if arch == "modepel":
         return StackDesc(family="modepel", width=int(cfg["width"]), vocab=int(cfg["vocab"]), layers=[_modepel_layer(i, l) for i, l in enumerate(cfg["layers"])],
                          compute_dtype=compute_dtype, max_seqs=max_seqs, max_ctx=max_ctx, budget_tokens=budget_tokens, norm_groups=1,

@@ -141,20 +141,72 @@ static bool load_vitudra_layer(const Json& L, size_t i, tgx_layer_desc& l, std::
   return true;
 }
 
+// one entry of a Zaluvik config's "layers": {"type": "attention" | "latent_attention", "mixer": {...}, "mlp": null | {"kind": "dense" | "moe", ...}}.
+// Attention: unit queries and keys, a sliding window, sigmoid weights with a per-head bias mixed across heads, a gate per output channel.  Latent attention:
+// rot_dim rotated dimensions beside dim per head, one rotated key part for all heads, a sliding window, softmax, a gate per head.  Dense feed-forwards use
+// the erf gelu; experts are chosen by sigmoid scores inside the best groups (a group counts as the sum of its two largest scores), weights normalised.
+static bool load_zaluvik_layer(const Json& L, size_t i, tgx_layer_desc& l, std::string& err) {
+  auto dim = [](const Json& j, const char* key) -> int32_t { const int64_t v = j.get_int(key, -1); return (v < 0 || v > ((int64_t)1 << 30)) ? -1 : (int32_t)v; };
+  const Json* mx = L.get("mixer");
+  const Json* ff = L.get("mlp");
+  const std::string type = L.get_str("type", "");
+  auto bad = [&](const std::string& what) { err = "config.json: layer " + std::to_string(i) + ": " + what; return false; };
+  if (!mx || mx->kind != Json::Obj) return bad("no mixer");
+  l.heads = dim(*mx, "heads"); l.dim = dim(*mx, "dim"); l.vdim = mx->has("vdim") ? dim(*mx, "vdim") : l.dim; l.scale = mx->get_float("scale", 1.f);
+  const Json* mask = mx->get("mask");
+  if (mask && mask->kind == Json::Obj) { l.mask_kind = TGX_MASK_WINDOW; l.mask_size = dim(*mask, "size"); }
+  if (type == "attention") {
+    l.mixer = TGX_MIXER_ATTENTION;
+    l.kv_heads = mx->has("kv_heads") ? dim(*mx, "kv_heads") : l.heads;
+    l.qk_norm = 1; l.score_fn = 1; l.head_mix = 1; l.gate_kind = 1;
+  } else if (type == "latent_attention") {
+    l.mixer = TGX_MIXER_LATENT_ATTENTION;
+    l.kv_rank = dim(*mx, "kv_rank"); l.rot_dim = mx->has("rot_dim") ? dim(*mx, "rot_dim") : 0; l.gate_kind = 2;
+    const Json* rot = mx->get("rot");
+    l.rot_dims = l.rot_dim; l.rot_base = 10000.f;
+    if (rot && rot->kind == Json::Obj) { if (rot->has("dims")) l.rot_dims = dim(*rot, "dims"); l.rot_base = rot->get_float("base", 10000.f); }
+    if (l.rot_dim <= 0) l.rot_dims = 0;
+  } else return bad("mixer '" + type + "' is not implemented");
+  if (!ff || ff->kind != Json::Obj) return true;
+  const std::string kind = ff->get_str("kind", "");
+  if (kind == "dense") { l.mlp = TGX_MLP_DENSE; l.ff = dim(*ff, "ff"); l.ff_act = 1; return true; }
+  const Json* ex = ff->get("expert");
+  const Json* ro = ff->get("router");
+  if (kind != "moe" || !ro || ro->kind != Json::Obj || !ex || ex->kind != Json::Obj) return bad("feed-forward kind '" + kind + "' is not implemented");
+  l.mlp = TGX_MLP_MOE;
+  l.experts = dim(*ro, "experts"); l.top = dim(*ro, "top"); l.ff = dim(*ex, "ff"); l.router_scale = 1.f;
+  l.router_fn = 1; l.group_score = 1; l.router_norm = 1;
+  const Json* gr = ro->get("groups");
+  l.groups = 1; l.groups_keep = 1;
+  if (gr && gr->kind == Json::Obj) { l.groups = dim(*gr, "count"); l.groups_keep = gr->has("keep") ? dim(*gr, "keep") : l.groups; }
+  const Json* sh = ff->get("shared");
+  l.shared_ff = sh && sh->kind == Json::Obj ? dim(*sh, "ff") : 0;
+  return true;
+}
+
 // config.json of a layered model: {"architecture": "Zakusun", "width", "vocab", "logit_scale", "norm": {"eps", "groups"}, "canon": {"taps"},
 // "layers": [{"type": mixer, "mixer": {heads, dim, vdim, kv_rank, scale}, "mlp": null | {"kind": "moe", "expert": {ff, limit}, "router": {experts, top}}}]}
 // or {"architecture": "Modepel", "width", "vocab", "norm": {"eps"}, "layers": [...]} with the layer entries of load_modepel_layer
 // or {"architecture": "Vitudra", "width", "vocab", "residual_mult", "norm": {"eps"}, "layers": [...]} with the layer entries of load_vitudra_layer
+// or {"architecture": "Zaluvik", "width", "vocab", "residual_mult", "embedding": {"scale"}, "loop": {"start", "stop", "times"}, "norm": {"eps"}, "layers": [...]}
+// with the layer entries of load_zaluvik_layer (logits against the embedding table)
 static bool load_stack_config(const Json& doc, const std::string& path, int compute_dtype, int max_batch, int max_ctx, int budget_tokens, ModelConfig& out, std::string& err) {
   const std::string arch = doc.get_str("architecture", "");
-  const bool vitudra = arch == "Vitudra", modepel = arch == "Modepel" || vitudra;      // (both: scalar-free config header, a separate head)
+  const bool vitudra = arch == "Vitudra", zaluvik = arch == "Zaluvik", modepel = arch == "Modepel" || vitudra || zaluvik;      // (all three: a config header without norm groups, taps and logit scale)
   if (arch != "Zakusun" && !modepel) { err = "Unsupported architecture: " + arch; return false; }
   auto dim = [](const Json& j, const char* key) -> int32_t { const int64_t v = j.get_int(key, -1); return (v < 0 || v > ((int64_t)1 << 30)) ? -1 : (int32_t)v; };
   out.layered = true;
-  out.model_type = vitudra ? "vitudra" : modepel ? "modepel" : "zakusun";
+  out.model_type = zaluvik ? "zaluvik" : vitudra ? "vitudra" : modepel ? "modepel" : "zakusun";
   tgx_stack_desc& s = out.stack;
-  s.family = vitudra ? TGX_FAMILY_VITUDRA : modepel ? TGX_FAMILY_MODEPEL : TGX_FAMILY_ZAKUSUN;
+  s.family = zaluvik ? TGX_FAMILY_ZALUVIK : vitudra ? TGX_FAMILY_VITUDRA : modepel ? TGX_FAMILY_MODEPEL : TGX_FAMILY_ZAKUSUN;
   s.residual_mult = doc.get_float("residual_mult", 1.f);
+  s.embed_scale = 1.f; s.loop_times = 1;
+  if (zaluvik) {
+    const Json* em = doc.get("embedding");
+    if (em && em->kind == Json::Obj) s.embed_scale = em->get_float("scale", 1.f);
+    const Json* lp = doc.get("loop");
+    if (lp && lp->kind == Json::Obj) { s.loop_start = dim(*lp, "start"); s.loop_stop = dim(*lp, "stop"); s.loop_times = dim(*lp, "times"); }
+  }
   s.width = dim(doc, "width"); s.vocab = dim(doc, "vocab"); s.compute_dtype = compute_dtype;
   s.max_seqs = max_batch < 1 ? 1 : max_batch;
   s.max_ctx = max_ctx > 0 ? max_ctx : 4096;
@@ -172,7 +224,7 @@ static bool load_stack_config(const Json& doc, const std::string& path, int comp
     const Json& L = layers->arr[i];
     tgx_layer_desc l{};
     if (modepel) {
-      if (!(vitudra ? load_vitudra_layer(L, i, l, err) : load_modepel_layer(L, i, l, err))) return false;
+      if (!(zaluvik ? load_zaluvik_layer(L, i, l, err) : vitudra ? load_vitudra_layer(L, i, l, err) : load_modepel_layer(L, i, l, err))) return false;
       out.layers.push_back(l);
       continue;
     }
@@ -193,7 +245,7 @@ static bool load_stack_config(const Json& doc, const std::string& path, int comp
   }
   s.layers = (int32_t)out.layers.size();
   tgx_model_desc& d = out.desc;
-  d.family = s.family; d.hidden = s.width; d.layers = s.layers; d.vocab = s.vocab; d.max_ctx = s.max_ctx; d.max_batch = s.max_seqs; d.compute_dtype = compute_dtype; d.tied = modepel ? 0 : 1;
+  d.family = s.family; d.hidden = s.width; d.layers = s.layers; d.vocab = s.vocab; d.max_ctx = s.max_ctx; d.max_batch = s.max_seqs; d.compute_dtype = compute_dtype; d.tied = modepel && !zaluvik ? 0 : 1;
   if (s.width <= 0 || s.vocab <= 0 || s.norm_groups <= 0 || s.canon_taps <= 0) { err = "config.json: width / vocab / norm.groups / canon.taps missing or out of range in " + path; return false; }
   return true;
 }
