@@ -229,7 +229,7 @@ typedef struct tgx_stack_desc {
   float residual_mult;    /* ABI 6, TGX_FAMILY_VITUDRA / ZALUVIK: the factor on what a sublayer adds to the stream */
   /* ABI 7, TGX_FAMILY_ZALUVIK */
   float embed_scale;      /* x = embed[token] * embed_scale                                         */
-  int32_t loop_start;     /* layers loop_start .. loop_stop - 1 run loop_times times (loop_times <= 1 or an empty span: no loop) */
+  int32_t loop_start;     /* layers loop_start .. loop_stop - 1 run loop_times times (an empty span: no loop) */
   int32_t loop_stop;
   int32_t loop_times;
 } tgx_stack_desc;

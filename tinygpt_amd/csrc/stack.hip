@@ -907,7 +907,7 @@ int create_affine_layers(tgx_ctx* c, const tgx_layer_desc* layers) {
   int rc;
   auto need = [&](const std::string& p, std::initializer_list<const char*> names) { for (const char* n : names) sm->missing.insert(p + n); };
   sm->missing.insert("final.norm.b");
-  const bool looped = d.loop_times > 1 && d.loop_stop > d.loop_start;
+  const bool looped = d.loop_times >= 1 && d.loop_stop > d.loop_start;      // (one pass still has the input product in front)
   if (looped) {
     if ((rc = dev_alloc(c, &sm->w_loop, W * 2 * W * es))) return rc;
     sm->missing.insert("loop.in");
@@ -1059,7 +1059,7 @@ int upload_affine(tgx_ctx* c, const char* name, const void* host, const int64_t*
 
 // what a layer-norm design's description may ask for
 int check_affine_desc(const tgx_stack_desc& d, const tgx_layer_desc* layers) {
-  if (d.loop_times > 1 && d.loop_stop > d.loop_start && (d.loop_start < 0 || d.loop_stop > d.layers)) return set_err(nullptr, TGX_ERR_INVALID, "loop %d .. %d outside the %d layers", d.loop_start, d.loop_stop, d.layers);
+  if (d.loop_times >= 1 && d.loop_stop > d.loop_start && (d.loop_start < 0 || d.loop_stop > d.layers)) return set_err(nullptr, TGX_ERR_INVALID, "loop %d .. %d outside the %d layers", d.loop_start, d.loop_stop, d.layers);
   for (int i = 0; i < d.layers; i++) {
     const tgx_layer_desc& l = layers[i];
     if (l.heads <= 0 || l.dim <= 0 || l.vdim <= 0) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: non-positive mixer size", i);

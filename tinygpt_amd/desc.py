@@ -418,7 +418,7 @@ class StackDesc:
 
     @property
     def looped(self) -> bool:
-        return self.loop_times > 1 and self.loop_stop > self.loop_start
+        return self.loop_times >= 1 and self.loop_stop > self.loop_start      # (a single pass still has the loop's input product in front)
 
     def layer_runs(self) -> "list[int]":
         """the layers in the order they run (a looped span repeats)"""
