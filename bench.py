@@ -84,7 +84,7 @@ def parse():
     ap.add_argument("--layered", default=None, metavar="SIZE[,SIZE]", help="instead of the headline: prefill and decode throughput of the layered (Zakusun) design at "
                     "layer sizes of real models (1b, 0.5b; random weights), beside a Llama-family model of the same width, depth and active parameters")
     ap.add_argument("--only", default="", help="with --layered: measure these models only (names before the size, with commas; for profiling one of them)")
-    ap.add_argument("--design", default="zakusun", choices=["zakusun", "modepel", "vitudra"], help="with --layered: which layered design is measured beside its closest relatives and the Llama-family model")
+    ap.add_argument("--design", default="zakusun", choices=["zakusun", "modepel", "vitudra", "zaluvik"], help="with --layered: which layered design is measured beside its closest relatives and the Llama-family model")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the cpu_baseline sample")
     return ap.parse_args()
 
@@ -356,6 +356,32 @@ def vitudra_desc(key, z, L, V, dtype, B, ctx):
                      name=f"vitudra-{key}", layers=layers)
 
 
+def zaluvik_desc(key, z, L, V, dtype, B, ctx):
+    """Zaluvik at the size of `z`: six layers of which the second and third run twice (eight layer runs, a cache per run) — windowed sigmoid attention with
+    mixed heads (grouped key / value heads of 128) and, at two places, windowed latent attention whose cached row is 448 latent + 64 rotated channels;
+    erf-gelu feed-forwards and sigmoid-routed experts (four groups, two kept, a shared expert) in turn"""
+    from tinygpt_amd.desc import LayerDesc, StackDesc
+    W = z["width"]
+    plan = ["attention", "attention", "latent_attention", "attention", "latent_attention", "attention"]
+    layers = []
+    for i, kind in enumerate(plan):
+        if kind == "attention":
+            l = LayerDesc(mixer="attention", heads=W // 128, kv_heads=max(1, W // 512), dim=128, vdim=128, scale=0.09, mask="window", mask_size=1024, qk_norm=True,
+                          score_fn="sigmoid", head_mix=True, gate_kind="channel")
+        else:
+            l = LayerDesc(mixer="latent_attention", heads=z["heads"], dim=z["dim"], vdim=z["vdim"], kv_rank=z["kv_rank"] - 64, rot_dim=64, rot_dims=64, rot_base=500000.0,
+                          scale=(z["dim"] + 64) ** -0.5, mask="window", mask_size=1024, gate_kind="head")
+        if i % 2 == 0:
+            l.mlp, l.ff, l.ff_act = "dense", z["top"] * z["ff"], "gelu"
+        else:
+            l.mlp, l.experts, l.top, l.ff, l.groups, l.groups_keep, l.shared_ff = "moe", z["experts"], z["top"], z["ff"], 4, 2, z["ff"]
+            l.router_fn, l.group_score, l.router_norm = "sigmoid", "top2", True
+        layers.append(l)
+    assert L == 8, "the plan above makes eight layer runs"
+    return StackDesc(family="zaluvik", width=W, vocab=V, compute_dtype=dtype, max_seqs=B, max_ctx=ctx, budget_tokens=B * (ctx + 64), norm_eps=1e-5, residual_mult=0.5,
+                     embed_scale=3.0, loop_start=1, loop_stop=3, loop_times=2, name=f"zaluvik-{key}", layers=layers)
+
+
 def layered_compare(args):
     from tinygpt_amd.desc import LayerDesc, ModelDesc, StackDesc
     from tinygpt_amd.ffi import GREEDY, Model
@@ -402,7 +428,8 @@ def layered_compare(args):
         ld = ModelDesc(family="llama", hidden=z["width"], layers=L, heads=z["llama"]["heads"], kv_heads=z["llama"]["kv_heads"], head_dim=z["width"] // z["llama"]["heads"],
                        inter=z["llama"]["inter"], vocab=V, max_ctx=ctx, tied=True, compute_dtype=args.dtype, norm_eps=1e-5, rope_theta=500000.0, max_batch=B, name=f"llama-{key}")
         todo = {"zakusun": [(sd, True)], "modepel": [(modepel_desc(key, z, L, V, args.dtype, B, ctx), True), (sd, True)],
-                "vitudra": [(vitudra_desc(key, z, L, V, args.dtype, B, ctx), True), (modepel_desc(key, z, L, V, args.dtype, B, ctx), True)]}[args.design] + [(ld, False)]
+                "vitudra": [(vitudra_desc(key, z, L, V, args.dtype, B, ctx), True), (modepel_desc(key, z, L, V, args.dtype, B, ctx), True)],
+                "zaluvik": [(zaluvik_desc(key, z, L, V, args.dtype, B, ctx), True), (modepel_desc(key, z, L, V, args.dtype, B, ctx), True), (sd, True)]}[args.design] + [(ld, False)]
         if args.only:
             todo = [t for t in todo if t[0].name.split("-")[0] in args.only.split(",")]
         for desc, layered in todo:

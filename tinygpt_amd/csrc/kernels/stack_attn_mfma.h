@@ -21,10 +21,11 @@ struct LatentMfmaArgs {
   const float* q;        // [T * heads][rank]
   const void* pool;      // [pages][page][rank]
   const void* poolT;     // [pages][rank][page]
-  const float* sink;     // [heads]
+  const float* sink;     // [heads] (nullptr: the softmax has no sink)
   float* out;            // [T * heads][rank]
   float* part; int nsplit, keys_per;      // keys_per: a multiple of 32
   int rank, heads, terms;
+  int mask_kind, mask_size;      // MASK_*: a row at position i sees the keys [first_key(i), i] (stack_meta.h); the walk starts at the key tile that holds the first row's first key
 };
 
 template <int DT, int NT, bool SPLIT>      // NT = rank / 128: 32-column output tiles per wave
@@ -40,8 +41,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(StepMeta m, Laten
   const int past = m.tok_pos[start];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, half = lane >> 5, l31 = lane & 31;
   const int kmax = past + min(r0 + 31, nrows - 1) / H + 1;      // keys of the tile's last row
-  int k0 = 0, k1 = kmax;
-  if (SPLIT) { k0 = min(kmax, (int)blockIdx.z * a.keys_per); k1 = min(kmax, k0 + a.keys_per); }
+  int k0 = first_key(past + r0 / H, a.mask_kind, a.mask_size) & ~31, k1 = kmax;
+  if (SPLIT) { k0 = min(kmax, k0 + (int)blockIdx.z * a.keys_per); k1 = min(kmax, k0 + a.keys_per); }
   const size_t row_base = (size_t)start * H;
   const int page = 1 << m.page_shift;
   const bf16_t* pool = reinterpret_cast<const bf16_t*>(a.pool);
@@ -75,7 +76,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(StepMeta m, Laten
   const int sr = r0 + srow;
   const bool svalid = sr < nrows;
   const int skeys = svalid ? past + sr / H + 1 : 0;
-  const bool sinked = svalid && (!SPLIT || blockIdx.z == 0);
+  const int sfirst = svalid ? first_key(skeys - 1, a.mask_kind, a.mask_size) : 0;
+  const bool sinked = a.sink && svalid && (!SPLIT || blockIdx.z == 0);
   float m_s = sinked ? a.sink[sr % H] : -INFINITY, l_s = sinked ? 1.f : 0.f;
 
   // operand fetches run one phase ahead: the score operands of the NEXT key tile are requested while this tile's softmax and P C run, the P C operands
@@ -123,7 +125,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(StepMeta m, Laten
 #pragma unroll
       for (int c = 0; c < 4; c++) {
         const float v = s_part[0][srow][kq + c] + s_part[1][srow][kq + c] + s_part[2][srow][kq + c] + s_part[3][srow][kq + c];
-        sv[c] = (kt + kq + c < min(skeys, k1)) ? v : -INFINITY;
+        sv[c] = (kt + kq + c < min(skeys, k1) && kt + kq + c >= sfirst) ? v : -INFINITY;
         tmax = fmaxf(tmax, sv[c]);
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 1, 64)); tmax = fmaxf(tmax, __shfl_xor(tmax, 2, 64)); tmax = fmaxf(tmax, __shfl_xor(tmax, 4, 64));
@@ -179,7 +181,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(StepMeta m, Laten
       const int ri = (r & 3) + 8 * (r >> 2) + 4 * half, gr = r0 + ri, col = wv * RQ + 32 * t + l31;
       if (gr >= nrows) continue;
       if (SPLIT) a.part[((row_base + gr) * a.nsplit + blockIdx.z) * (size_t)(a.rank + 2) + 2 + col] = acc[t][r];
-      else a.out[(row_base + gr) * a.rank + col] = acc[t][r] / s_l[ri];
+      else a.out[(row_base + gr) * a.rank + col] = s_l[ri] > 0.f ? acc[t][r] / s_l[ri] : 0.f;
     }
 }
 

@@ -87,8 +87,8 @@ __global__ __launch_bounds__(256) void affine_seam_kernel(AffineSeamArgs a) {
 //   out_h(i) = sum_j w'_h(i, j) v_kv(h)(j)                             head h keeps its own key / value head
 // and out_h is multiplied by sigmoid(gate) per channel where a gate is given.  Every key, also those of the step's own tokens, is read from the pool.
 // One workgroup per token (and per share of its keys in the split form).  Keys are taken KT at a time:
-//   scores   a thread owns one key of the tile: its key row against every head's query (queries in LDS, read as broadcasts), sigmoid
-//   mix      the same thread mixes its key's `heads` weights (its own column of the LDS tile: no exchange between threads)
+//   scores   the tile's (key, head) pairs are dealt to the threads: a key row against the head's query (queries in LDS, read as broadcasts), sigmoid
+//   mix      the pairs again: a pair's mixed weight from its key's `heads` weights in LDS
 //   values   a thread owns NPT output channels (head, c): it walks the tile's keys, reading weights from LDS and value rows coalesced from the pool
 // Nothing is normalised, so the shares of a divided window are simply added (sigmoid_mix_merge_kernel, in split order).
 struct MixAttnArgs {
@@ -131,44 +131,44 @@ __global__ __launch_bounds__(256) void sigmoid_mix_attn_kernel(StepMeta m, MixAt
   }
   for (int kb = k0; kb < k1; kb += KT) {
     const int nk = min(KT, k1 - kb);
-    __syncthreads();                         // queries staged; the previous tile's weights have been read
+    __syncthreads();                         // queries staged; the previous tile's weights and rows have been read
     if (tid < nk) {
       const int j = kb + tid;
       const int page = m.tbl[(size_t)row * m.tbl_stride + (j >> m.page_shift)];
-      const int slot = (page << m.page_shift) + (j & pmask);
-      s_slot[tid] = slot;
-      const elem_t<DT>* kr = pk + (size_t)slot * kd;
-      for (int c = 0; c < G; c++) {
-        const elem_t<DT>* kc = kr + (size_t)c * a.dim;
-        for (int g = c * qpg; g < (c + 1) * qpg; g++) {
-          const float* qg = s_q + (size_t)g * a.dim;
-          float s = 0.f;
-          if (VEC) {
-            for (int d = 0; d < a.dim; d += 8) {
-              float f[8];
-              slice_unpack<DT>(load_slice<DT>(kc, (size_t)(d >> 3)), f);
-              const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + d), qb = *reinterpret_cast<const f32x4*>(qg + d + 4);
-#pragma unroll
-              for (int e = 0; e < 4; e++) s = fmaf(qa[e], f[e], s);
-#pragma unroll
-              for (int e = 0; e < 4; e++) s = fmaf(qb[e], f[4 + e], s);
-            }
-          } else {
-            for (int d = 0; d < a.dim; d++) s = fmaf(qg[d], elem_to_f32<DT>(kc[d]), s);
-          }
-          s = fmaf(s, a.scale, a.pb ? a.pb[g] : 0.f);
-          s_w[(size_t)g * KT + tid] = 1.0f / (1.0f + expf(-s));
-        }
-      }
-      if (a.talk) {
-        for (int h = 0; h < H; h++) {
-          float v = 0.f;
-          for (int g = 0; g < H; g++) v = fmaf(s_t[h * H + g], s_w[(size_t)g * KT + tid], v);
-          s_w2[(size_t)h * KT + tid] = v;
-        }
-      }
+      s_slot[tid] = (page << m.page_shift) + (j & pmask);
     }
     __syncthreads();
+    for (int i = tid; i < nk * H; i += 256) {      // scores: one (key, head) pair per thread and round; neighbours take neighbouring keys of one head
+      const int g = i / nk, jj = i - g * nk;
+      const elem_t<DT>* kc = pk + (size_t)s_slot[jj] * kd + (size_t)(g / qpg) * a.dim;
+      const float* qg = s_q + (size_t)g * a.dim;
+      float s = 0.f;
+      if (VEC) {
+        for (int d = 0; d < a.dim; d += 8) {
+          float f[8];
+          slice_unpack<DT>(load_slice<DT>(kc, (size_t)(d >> 3)), f);
+          const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + d), qb = *reinterpret_cast<const f32x4*>(qg + d + 4);
+#pragma unroll
+          for (int e = 0; e < 4; e++) s = fmaf(qa[e], f[e], s);
+#pragma unroll
+          for (int e = 0; e < 4; e++) s = fmaf(qb[e], f[4 + e], s);
+        }
+      } else {
+        for (int d = 0; d < a.dim; d++) s = fmaf(qg[d], elem_to_f32<DT>(kc[d]), s);
+      }
+      s = fmaf(s, a.scale, a.pb ? a.pb[g] : 0.f);
+      s_w[(size_t)g * KT + jj] = 1.0f / (1.0f + expf(-s));
+    }
+    __syncthreads();
+    if (a.talk) {
+      for (int i = tid; i < nk * H; i += 256) {    // mix: every (key, head) pair reads its key's weights of all heads
+        const int h = i / nk, jj = i - h * nk;
+        float v = 0.f;
+        for (int g = 0; g < H; g++) v = fmaf(s_t[h * H + g], s_w[(size_t)g * KT + jj], v);
+        s_w2[(size_t)h * KT + jj] = v;
+      }
+      __syncthreads();
+    }
     const float* sw = a.talk ? s_w2 : s_w;
     for (int jj = 0; jj < nk; jj++) {
       const elem_t<DT>* vr = pv + (size_t)s_slot[jj] * vd;

@@ -61,6 +61,8 @@ struct StackRun {
   bool inject = false;          // x <- W_loop [x; x0] in front of this run (the first layer of a pass of the loop)
   ebyte* pool = nullptr;        // attention: keys [pages][page_tokens][kv_heads * dim]; latent attention: [pages][page_tokens][kv_rank + rot_dim]
   ebyte* poolV = nullptr;       // attention: values [pages][page_tokens][kv_heads * vdim]
+  ebyte* poolT = nullptr;       // the transposed copy for the matrix-core kernels (runs that take them): a latent run's rows [pages][kv_rank + rot_dim][page_tokens],
+                                // an attention run's values [pages][kv_heads * vdim][page_tokens]
 };
 
 struct RotTable { int dims; float base; float factor; float* cs; };      // cos / sin of (position, pair) [max_ctx][dims / 2][2], angle = position * base^(-2 pair / dims) / factor, made on the host in double precision

@@ -711,12 +711,11 @@ void launch_mix_attn_t(tgx_ctx* c, const tgx::StepMeta& m, const tgx::MixAttnArg
 }
 constexpr int MIX_ATTN_MAX_OUT = 32 * 256;            // heads * vdim of the sigmoid attention (output channels per thread <= 32)
 constexpr size_t MIX_ATTN_MAX_LDS = 144 * 1024;
-int mix_attn_tile_keys(int heads, int dim) {          // keys per tile: as many as keep the workgroup's LDS within 64 KB, 64 at least
-  for (int kt = 256; kt > 64; kt >>= 1) if (tgx::mix_attn_lds_bytes(heads, dim, kt) <= 64 * 1024) return kt;
-  return 64;
+int mix_attn_tile_keys(int heads, int dim) {          // keys per tile: 64, or 32 where that keeps the workgroup's LDS within 64 KB
+  return tgx::mix_attn_lds_bytes(heads, dim, 64) <= 64 * 1024 ? 64 : 32;
 }
 
-int run_affine_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const StackRun& run, int T, int max_keys) {
+int run_affine_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const StackRun& run, int T, int S, int max_keys, int max_count) {
   StackModel* sm = c->stack;
   const tgx_layer_desc& ld = w.d;
   const int W = sm->d.width, H = ld.heads, G = ld.kv_heads, qd = H * ld.dim, kd = G * ld.dim, kvv = G * ld.vdim, vd = H * ld.vdim, nin = qd + kd + kvv + vd;
@@ -737,11 +736,12 @@ int run_affine_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, con
   const bool vec = ld.dim % 8 == 0;
   const int span = ld.mask_kind == tgx::MASK_CAUSAL ? max_keys : std::min(max_keys, ld.mask_size);
   int nsplit = 1;
-  if (span >= sm->gqa_split_min_keys && (long long)T < c->num_cus) {      // few tokens and a long span: the keys are divided between workgroups, whole tiles each
+  if (span >= std::min(sm->gqa_split_min_keys, 128) && (long long)T < c->num_cus) {      // few tokens and a long span: the keys are divided between workgroups
     nsplit = (int)std::min<long long>(64, (2LL * c->num_cus) / T);
-    const int per = std::max(aa.kt, ((span + nsplit - 1) / nsplit + aa.kt - 1) / aa.kt * aa.kt);
+    const int per = std::max(32, ((span + nsplit - 1) / nsplit + 31) / 32 * 32);
     nsplit = (span + per - 1) / per;
     aa.keys_per = per;
+    aa.kt = std::min(aa.kt, per);
   }
   if (nsplit > 1) {
     int rc = ensure_part(c, (size_t)T * nsplit * (size_t)vd);
@@ -761,7 +761,7 @@ int run_affine_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, con
 
 // latent attention with a rotated key part that all heads share and a window: the pool row is [normed latent | rotated key part]; every head's query is
 // taken into that space ([scale W_uk^T q_plain | scale rot(q_rot)]), so a score is one dot product with the cached row and nothing else is cached
-int run_affine_latent(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const StackRun& run, int T, int max_keys) {
+int run_affine_latent(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const StackRun& run, int T, int S, int max_keys, int max_count) {
   StackModel* sm = c->stack;
   const tgx_layer_desc& ld = w.d;
   const int W = sm->d.width, H = ld.heads, qs = ld.dim + ld.rot_dim, qd = H * qs, R = ld.kv_rank, RR = R + ld.rot_dim, vd = H * ld.vdim, ng = ld.gate_kind == 2 ? H : vd, nin = qd + RR + ng;
@@ -769,7 +769,7 @@ int run_affine_latent(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const 
   g.A = sm->a; g.lda = W; g.B = w.w_in; g.ldb = W; g.C = sm->proj; g.ldc = nin; g.M = T; g.N = nin; g.K = W; g.scale = 1.f;
   launch_gemm(c, g, tgx::SG_STORE, 1);
   tgx::LatentAppendArgs la{};
-  la.src = sm->proj; la.lds = nin; la.col0 = qd; la.nw = w.lat_norm; la.pool = run.pool; la.rank = R; la.eps = sm->d.norm_eps;
+  la.src = sm->proj; la.lds = nin; la.col0 = qd; la.nw = w.lat_norm; la.pool = run.pool; la.poolT = run.poolT; la.rank = R; la.eps = sm->d.norm_eps;
   la.rot_dim = ld.rot_dim; la.rot_dims = ld.rot_dims; la.cs = w.rot >= 0 ? sm->rot[(size_t)w.rot].cs : nullptr;
   la.q = sm->proj; la.heads = H; la.qstride = qs; la.qoff = ld.dim; la.qscale = ld.scale; la.ql = sm->ql;
   TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::latent_append_kernel<DT>, dim3(T), dim3(64), 0, c->stream, m, la))
@@ -781,9 +781,32 @@ int run_affine_latent(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const 
   tgx::LatentAttnArgs aa{};
   aa.q = sm->ql; aa.ldq = (long long)H * RR; aa.pool = run.pool; aa.sink = nullptr; aa.out = sm->lat; aa.ldo = (long long)H * RR; aa.rank = RR; aa.heads = H;
   aa.mask_kind = ld.mask_kind; aa.mask_size = ld.mask_size;
-  const int span = ld.mask_kind == tgx::MASK_CAUSAL ? max_keys : std::min(max_keys, ld.mask_size);
+  const int span = ld.mask_kind == tgx::MASK_CAUSAL ? max_keys : std::min(max_keys, ld.mask_size + 64);      // (the matrix-core kernel starts at a key tile's edge and a row tile spans up to 32 tokens)
   int nsplit = 1;
-  if (span >= sm->attn_split_min_keys && (long long)T * H < 2LL * c->num_cus) {
+  if (run.poolT && sm->attn_mfma) {
+    // rows = (token, head) pairs of an entry in tiles of 32; few tiles and a long span: the keys are divided between workgroups
+    tgx::LatentMfmaArgs ma{};
+    ma.q = sm->ql; ma.pool = run.pool; ma.poolT = run.poolT; ma.sink = nullptr; ma.out = sm->lat; ma.rank = RR; ma.heads = H; ma.terms = c->act16 ? 1 : 2;
+    ma.mask_kind = ld.mask_kind; ma.mask_size = ld.mask_size;
+    const int tiles = (max_count * H + 31) / 32;
+    if (span >= std::min(sm->attn_split_min_keys, 256) && (long long)tiles * S < c->num_cus) {
+      nsplit = (int)std::min<long long>(64, (2LL * c->num_cus) / ((long long)tiles * S));
+      const int per = std::max(64, ((span + nsplit - 1) / nsplit + 31) / 32 * 32);      // two key tiles per workgroup at least
+      nsplit = (span + per - 1) / per;
+      ma.keys_per = per;
+    }
+    if (nsplit > 1) {
+      int rc = ensure_part(c, (size_t)T * H * nsplit * (size_t)(RR + 2));
+      if (rc) return rc;
+      ma.part = sm->part; ma.nsplit = nsplit;
+      aa.part = sm->part; aa.nsplit = nsplit;
+      if (c->dt == tgx::DT_F16) launch_attn_mfma_t<tgx::DT_F16, true>(c, m, ma, dim3(tiles, S, nsplit)); else launch_attn_mfma_t<tgx::DT_BF16, true>(c, m, ma, dim3(tiles, S, nsplit));
+      hipLaunchKernelGGL(tgx::latent_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, aa);
+    } else {
+      if (c->dt == tgx::DT_F16) launch_attn_mfma_t<tgx::DT_F16, false>(c, m, ma, dim3(tiles, S)); else launch_attn_mfma_t<tgx::DT_BF16, false>(c, m, ma, dim3(tiles, S));
+    }
+  } else {
+  if (span >= std::min(sm->attn_split_min_keys, 512) && (long long)T * H < 2LL * c->num_cus) {
     nsplit = (int)std::min<long long>(64, (4LL * c->num_cus) / ((long long)T * H));
     const int per = std::max(256, ((span + nsplit - 1) / nsplit + 63) / 64 * 64);
     nsplit = (span + per - 1) / per;
@@ -797,6 +820,7 @@ int run_affine_latent(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const 
     hipLaunchKernelGGL(tgx::latent_attn_merge_kernel, dim3(T, H), dim3(256), 0, c->stream, aa);
   } else {
     TGX_DT_SWITCH(c->dt, (launch_attn_t<DT, false>(c, m, aa, dim3(T, H))))
+  }
   }
   // o[t][h] = (lat[t][h][0 .. R) . uv[h]^T) * sigmoid(gate of the head, or of the channel)
   g = tgx::StackGemmArgs{};
@@ -854,7 +878,7 @@ void run_affine_ff(tgx_ctx* c, StackLayerW& w, int T) {
   }
 }
 
-int run_layers_affine(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys) {
+int run_layers_affine(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int max_count) {
   StackModel* sm = c->stack;
   const tgx::StepMeta m = step_meta(sm, mp, T, S);
   const int W = sm->d.width;
@@ -876,7 +900,7 @@ int run_layers_affine(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys
       normed = false;
     }
     if (!normed) hipLaunchKernelGGL(tgx::layer_norm_rows_kernel, dim3(T), dim3(256), 0, c->stream, sm->x, nullptr, ln, ln + W, sm->a, W, eps);
-    int rc = ld.mixer == TGX_MIXER_ATTENTION ? run_affine_attention(c, m, w, run, T, max_keys) : run_affine_latent(c, m, w, run, T, max_keys);
+    int rc = ld.mixer == TGX_MIXER_ATTENTION ? run_affine_attention(c, m, w, run, T, S, max_keys, max_count) : run_affine_latent(c, m, w, run, T, S, max_keys, max_count);
     if (rc) return rc;
     const bool last = ri + 1 == sm->runs.size();
     const bool next_direct = !last && !sm->runs[ri + 1].inject;      // the next run's first norm can ride in this run's last seam
@@ -1067,7 +1091,7 @@ int check_affine_desc(const tgx_stack_desc& d, const tgx_layer_desc* layers) {
     if (l.mixer == TGX_MIXER_ATTENTION) {
       if (l.kv_heads <= 0 || l.heads % l.kv_heads) return set_err(nullptr, TGX_ERR_INVALID, "layer %d: %d query heads over %d key / value heads", i, l.heads, l.kv_heads);
       if (l.score_fn != 1) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: this family's attention takes sigmoid weights (score_fn 1)", i);
-      if ((long long)l.heads * l.vdim > MIX_ATTN_MAX_OUT || tgx::mix_attn_lds_bytes(l.heads, l.dim, 64) > MIX_ATTN_MAX_LDS)
+      if ((long long)l.heads * l.vdim > MIX_ATTN_MAX_OUT || tgx::mix_attn_lds_bytes(l.heads, l.dim, 32) > MIX_ATTN_MAX_LDS)
         return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: sigmoid attention: %d heads of %d / %d exceed the kernel's %d output channels or its LDS", i, l.heads, l.dim, l.vdim, MIX_ATTN_MAX_OUT);
       if (l.gate_kind != 0 && l.gate_kind != 1) return set_err(nullptr, TGX_ERR_UNSUPPORTED, "layer %d: attention gates are per channel", i);
     } else if (l.mixer == TGX_MIXER_LATENT_ATTENTION) {
@@ -1089,7 +1113,7 @@ int check_affine_desc(const tgx_stack_desc& d, const tgx_layer_desc* layers) {
 }
 
 int run_layers(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys, int max_count) {
-  if (c->stack->affine) return run_layers_affine(c, mp, T, S, max_keys);
+  if (c->stack->affine) return run_layers_affine(c, mp, T, S, max_keys, max_count);
   if (c->stack->joint) return run_layers_joint(c, mp, T, S, max_keys, max_count);
   return c->stack->sandwich ? run_layers_sandwich(c, mp, T, S, max_keys, max_count) : run_layers_latent(c, mp, T, S, max_keys, max_count);
 }
@@ -1708,6 +1732,11 @@ int stack_finalize(tgx_ctx* c) {
       const size_t pe = rows * (size_t)(l.kv_rank + l.rot_dim) * c->esz;
       if ((rc = dev_alloc(c, &run.pool, pe))) return rc;
       HIP_OK(c, hipMemset(run.pool, 0, pe));
+      tgx_layer_desc row = l; row.kv_rank = l.kv_rank + l.rot_dim;      // the matrix-core kernel sees the cached row, latent and rotated part, as one latent
+      if (layer_attn_mfma(c, row)) {
+        if ((rc = dev_alloc(c, &run.poolT, pe))) return rc;
+        HIP_OK(c, hipMemset(run.poolT, 0, pe));
+      }
     }
   }
   for (auto& w : sm->L) {
@@ -1830,7 +1859,7 @@ void stack_destroy(tgx_ctx* c) {
     fr(w.b_in); fr(w.poolV); fr(w.poolVT); fr(w.vmix); fr(w.head_w); fr(w.mS); fr(w.mn); fr(w.mm); fr(w.act); fr(w.ws_gate); fr(w.ws_up); fr(w.ws_down);
   }
   for (auto& r : sm->rot) fr(r.cs);
-  for (auto& r : sm->runs) { fr(r.pool); fr(r.poolV); }
+  for (auto& r : sm->runs) { fr(r.pool); fr(r.poolV); fr(r.poolT); }
   for (auto& w : sm->L) { fr(w.ln); fr(w.talk); fr(w.pb); }
   fr(sm->w_loop); fr(sm->xcat);
   fr(sm->mixed); fr(sm->lora); fr(sm->rec_in);
