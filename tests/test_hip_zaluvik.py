@@ -453,3 +453,39 @@ def test_what_the_library_refuses():
     with pytest.raises(TgxError, match="l0.mix.talk"):
         m.finalize()
     m.close()
+
+
+# ---- attention on the matrix cores (16-bit storage) ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("size", [1, 33, 64, 100, 0])
+@pytest.mark.parametrize("kind,shape", [("attention", dict(heads=4, kv_heads=1, dim=64, vdim=32)), ("attention", dict(heads=8, kv_heads=2, dim=128, vdim=128)),
+                                        ("attention", dict(heads=6, kv_heads=3, dim=48, vdim=96)), ("attention", dict(heads=3, kv_heads=3, dim=16, vdim=64)),
+                                        ("attention", dict(heads=16, kv_heads=2, dim=32, vdim=32)),
+                                        ("latent", dict(heads=4, dim=24, rot_dim=32, vdim=40, kv_rank=96)), ("latent", dict(heads=16, dim=64, rot_dim=64, vdim=64, kv_rank=192)),
+                                        ("latent", dict(heads=3, dim=32, rot_dim=0, vdim=32, kv_rank=128))])
+def test_matrix_core_attention_equals_the_lane_kernels(kind, shape, size):
+    """the same bf16 weights and cached rows through both forms of each attention, under windows that start inside a key tile: portions whose 32-row tiles
+    cut through tokens and windows, a mixed batch, decoding, contexts across page borders, and divided windows"""
+    mask = {"size": size} if size else None
+    mk_layer = attn if kind == "attention" else lat
+    scale = 2.0 if kind == "attention" else 0.2
+    cfg = config([mk_layer(dense(), mask=mask, scale=scale, **shape), mk_layer(mask={"size": size + 7} if size else None, scale=scale, **shape)], width=64, loop=(0, 1, 2))
+    w = zo.random_tensors(cfg, shape["heads"])
+    tens = {k: np.asarray(v, np.float32) for k, v in w.items()}
+    mk = lambda: SlotEngine(desc=stack_desc_from_config(cfg, "bf16", max_seqs=4, max_ctx=1024, budget_tokens=2048), tensors=tens)
+    fast, slow = mk(), mk()
+    slow.model.set_option("attn.mfma", 0)
+    a, b, c = tokens(cfg, 200, 1), tokens(cfg, 75, 2), tokens(cfg, 9, 3)
+    want = want_of(cfg, w, a)[[0, 1, 69, 130, 131, 199]]
+    outs = []
+    for eng in (fast, slow):
+        o = [eng.step([("a", a[:70], [0, 1, 69]), ("b", b[:3], [2])])]
+        o.append(eng.step([("a", a[70:131], [60]), ("c", c, [8]), ("b", b[3:4], [0])]))
+        o.append(eng.step([("b", b[4:], [70]), ("a", a[131:132], [0])]))
+        o.append(eng.step([("a", a[132:199], [])]))
+        eng.model.set_option("attn.split_min", 64)
+        o.append(eng.step([("a", a[199:], [0]), ("b", [5], [0])]))
+        outs.append(np.concatenate(o))
+    assert np.abs(outs[0] - outs[1]).max() / np.abs(outs[1]).max() < 1e-3
+    check(outs[0][[0, 1, 2, 4, 8, 9]], want, "bf16")               # a's positions 0, 1, 69, 130, 131, 199 in the order the steps returned them
+    check(outs[0][[6, 7]], want_of(cfg, w, b)[[3, 74]], "bf16")
+    fast.close(); slow.close()

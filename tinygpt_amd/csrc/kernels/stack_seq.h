@@ -118,6 +118,7 @@ struct GqaAppendArgs {
   int rot_pairs;             // 1: neighbours turn together
   float q_temp_coef; int q_temp_every;      // coef 0: no query temperature
   float qk_unit_eps;         // > 0: every q and k head is first divided by sqrt(mean(head^2) + qk_unit_eps) (no weight)
+  unsigned short *q_hi, *q_lo;      // [T][heads * dim] (nullptr: not kept): the finished queries as two 16-bit terms, the A operand of a matrix-core score product
 };
 template <int DT>
 __global__ __launch_bounds__(256) void gqa_append_kernel(StepMeta m, GqaAppendArgs a) {
@@ -149,6 +150,13 @@ __global__ __launch_bounds__(256) void gqa_append_kernel(StepMeta m, GqaAppendAr
     __syncthreads();
     const float f = fmaf(a.q_temp_coef, logf((float)((pos + 1) / a.q_temp_every) + 1.0f), 1.0f);
     for (int c = threadIdx.x; c < a.heads * a.dim; c += 256) row[c] *= f;
+  }
+  if constexpr (DT != DT_F32) {
+    if (a.q_hi) {
+      __syncthreads();
+      const size_t qd = (size_t)a.heads * a.dim;
+      for (int c = threadIdx.x; c < (int)qd; c += 256) split16<DT>(row[c], a.q_hi[(size_t)t * qd + c], a.q_lo[(size_t)t * qd + c]);
+    }
   }
   if (!a.poolK) return;
   __syncthreads();

@@ -79,6 +79,8 @@ struct StackModel {
   std::vector<StackRun> runs;          // affine designs: the layers in the order they run
   ebyte* w_loop = nullptr;             // [width][2 width]: the loop's input product on [x; x0]
   float* xcat = nullptr;               // step workspace [T][2 width]: the stream beside the embedding output
+  unsigned short* qplanes = nullptr;   // step workspace [2][T][max_qd]: an attention layer's queries as two 16-bit terms (matrix-core score products)
+  int max_qd = 0;
   float *mixed = nullptr, *lora = nullptr, *rec_in = nullptr;      // joint designs' step workspace: the token-shift mixes, the decay's inner product, the delta rule's inputs
   int max_shift = 0, max_lora = 0, max_rec = 0;
   ebyte* head = nullptr;               // [vocab][width] (sandwich and joint designs; the others multiply by the embedding table)

@@ -172,7 +172,7 @@ int ensure_ws(tgx_ctx* c, int T) {
   auto fr = [](auto*& p) { if (p) (void)hipFree(p); p = nullptr; };
   fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw); fr(sm->yh); fr(sm->yd); fr(sm->xn); fr(sm->lg);
   fr(sm->sel); fr(sm->perm); fr(sm->ptok); fr(sm->tile_e); fr(sm->tile_m0); fr(sm->meta_dev); fr(sm->zr);
-  fr(sm->a2); fr(sm->ytmp); fr(sm->ysh); fr(sm->sgw); fr(sm->vfirst); fr(sm->hs); fr(sm->mixed); fr(sm->lora); fr(sm->rec_in); fr(sm->xcat);
+  fr(sm->a2); fr(sm->ytmp); fr(sm->ysh); fr(sm->sgw); fr(sm->vfirst); fr(sm->hs); fr(sm->mixed); fr(sm->lora); fr(sm->rec_in); fr(sm->xcat); fr(sm->qplanes);
   if (sm->meta_host) { (void)hipHostFree(sm->meta_host); sm->meta_host = nullptr; }
   const int cap = std::max(T, 64);
   const size_t W = (size_t)sm->d.width, n = (size_t)cap;
@@ -181,7 +181,8 @@ int ensure_ws(tgx_ctx* c, int T) {
     if ((rc = dev_alloc(c, &sm->a2, n * W)) || (rc = dev_alloc(c, &sm->ytmp, n * W)) || (rc = dev_alloc(c, &sm->ysh, n * W)) || (rc = dev_alloc(c, &sm->sgw, n)) ||
         (rc = dev_alloc(c, &sm->vfirst, n * (size_t)std::max(1, sm->max_kvv))) || (rc = dev_alloc(c, &sm->hs, n * (size_t)std::max(1, sm->max_hv)))) return rc;
   } else if (sm->affine) {   // the seam's scratch row, the shared expert's row, the stream beside the embedding output
-    if ((rc = dev_alloc(c, &sm->ytmp, n * W)) || (rc = dev_alloc(c, &sm->ysh, n * W)) || (rc = dev_alloc(c, &sm->xcat, 2 * n * W))) return rc;
+    if ((rc = dev_alloc(c, &sm->ytmp, n * W)) || (rc = dev_alloc(c, &sm->ysh, n * W)) || (rc = dev_alloc(c, &sm->xcat, 2 * n * W)) ||
+        (rc = dev_alloc(c, &sm->qplanes, 2 * n * (size_t)std::max(1, sm->max_qd) + 8))) return rc;
   } else if (sm->joint) {    // the recurrent mixers' side buffers: un-normed outputs, token-shift mixes, the decay's inner product, the delta rule's inputs
     if ((rc = dev_alloc(c, &sm->hs, n * (size_t)std::max(1, sm->max_hv))) || (rc = dev_alloc(c, &sm->mixed, n * (size_t)std::max(1, sm->max_shift))) ||
         (rc = dev_alloc(c, &sm->lora, n * (size_t)std::max(1, sm->max_lora))) || (rc = dev_alloc(c, &sm->rec_in, n * (size_t)std::max(1, sm->max_rec)))) return rc;
@@ -715,6 +716,30 @@ int mix_attn_tile_keys(int heads, int dim) {          // keys per tile: 64, or 3
   return tgx::mix_attn_lds_bytes(heads, dim, 64) <= 64 * 1024 ? 64 : 32;
 }
 
+// the matrix-core form of the sigmoid attention serves 16-bit storage, key sizes in steps of 16, value sizes in steps of 32 up to 128, 1 / 2 / 4 / 8 query
+// heads per key / value head and pages of a multiple of 32 tokens
+constexpr int MIX_MFMA_MIN_COUNT = 16;      // portions from this many tokens on take it; shorter ones (and decoded tokens) the lane kernel
+bool layer_mix_mfma(const tgx_ctx* c, const tgx_layer_desc& l) {
+  const int qpg = l.kv_heads > 0 ? l.heads / l.kv_heads : 0;
+  return c->dt != tgx::DT_F32 && l.dim % 16 == 0 && l.vdim % 32 == 0 && l.vdim <= 128 && (qpg == 1 || qpg == 2 || qpg == 4 || qpg == 8) && c->stack->page_shift >= 5 &&
+         tgx::mix_mfma_lds_bytes(l.heads, qpg) <= MIX_ATTN_MAX_LDS;
+}
+template <int DT>
+void launch_mix_mfma_t(tgx_ctx* c, const tgx::StepMeta& m, const tgx::MixMfmaArgs& a, dim3 grid) {
+  const int qpg = a.heads / a.kv_heads;
+  const size_t lds = tgx::mix_mfma_lds_bytes(a.heads, qpg);
+  auto go = [&](auto Q) {
+    constexpr int QPG = decltype(Q)::value;
+    auto* fn = &tgx::sigmoid_mix_mfma_kernel<DT, QPG>;
+    if (lds > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(fn, grid, dim3(256), lds, c->stream, m, a);
+  };
+  if (qpg == 1) go(std::integral_constant<int, 1>{});
+  else if (qpg == 2) go(std::integral_constant<int, 2>{});
+  else if (qpg == 4) go(std::integral_constant<int, 4>{});
+  else go(std::integral_constant<int, 8>{});
+}
+
 int run_affine_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const StackRun& run, int T, int S, int max_keys, int max_count) {
   StackModel* sm = c->stack;
   const tgx_layer_desc& ld = w.d;
@@ -726,7 +751,22 @@ int run_affine_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, con
   tgx::GqaAppendArgs ap{};
   ap.proj = sm->proj; ap.ldp = nin; ap.heads = H; ap.kv_heads = G; ap.dim = ld.dim; ap.vdim = ld.vdim; ap.poolK = run.pool; ap.poolV = run.poolV;
   ap.qk_unit_eps = ld.qk_norm ? sm->d.norm_eps : 0.f;
+  const bool mfma = run.poolT && sm->attn_mfma && max_count >= MIX_MFMA_MIN_COUNT;
+  ap.poolVT = run.poolT;
+  if (mfma) { ap.q_hi = sm->qplanes; ap.q_lo = sm->qplanes + (((size_t)sm->cap_tokens * sm->max_qd + 7) & ~(size_t)7); }      // (both planes 16-byte aligned)
   TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::gqa_append_kernel<DT>, dim3(T), dim3(256), 0, c->stream, m, ap))
+  if (mfma) {
+    tgx::MixMfmaArgs ma{};
+    ma.qh = ap.q_hi; ma.ql = ap.q_lo; ma.poolK = run.pool; ma.poolVT = run.poolT; ma.pb = w.pb; ma.talk = ld.head_mix ? w.talk : nullptr;
+    ma.gate = ld.gate_kind == 1 ? sm->proj + qd + kd + kvv : nullptr; ma.ldg = nin; ma.out = sm->o; ma.ldo = vd;
+    ma.heads = H; ma.kv_heads = G; ma.dim = ld.dim; ma.vdim = ld.vdim; ma.terms = c->act16 ? 1 : 2; ma.scale = ld.scale; ma.mask_kind = ld.mask_kind; ma.mask_size = ld.mask_size;
+    const dim3 grid((max_count + 31) / 32, S, G);
+    if (c->dt == tgx::DT_F16) launch_mix_mfma_t<tgx::DT_F16>(c, m, ma, grid); else launch_mix_mfma_t<tgx::DT_BF16>(c, m, ma, grid);
+    tgx::StackGemmArgs go{};
+    go.A = sm->o; go.lda = vd; go.B = w.w_o; go.ldb = vd; go.C = sm->yd; go.ldc = W; go.M = T; go.N = W; go.K = vd; go.scale = 1.f;
+    launch_gemm(c, go, tgx::SG_STORE, 1);
+    return TGX_OK;
+  }
   tgx::MixAttnArgs aa{};
   aa.q = sm->proj; aa.ldq = nin; aa.poolK = run.pool; aa.poolV = run.poolV; aa.pb = w.pb; aa.talk = ld.head_mix ? w.talk : nullptr;
   aa.gate = ld.gate_kind == 1 ? sm->proj + qd + kd + kvv : nullptr; aa.ldg = nin; aa.out = sm->o; aa.ldo = vd;
@@ -958,6 +998,7 @@ int create_affine_layers(tgx_ctx* c, const tgx_layer_desc* layers) {
     if (l.mixer == TGX_MIXER_ATTENTION) {
       const size_t qd = H * l.dim, kd = (size_t)l.kv_heads * l.dim, kvv = (size_t)l.kv_heads * l.vdim;
       nin = qd + kd + kvv + vd;
+      sm->max_qd = std::max(sm->max_qd, (int)qd);
       if ((rc = dev_alloc(c, &w.talk, H * H)) || (rc = dev_alloc(c, &w.pb, H))) return rc;
       HIP_OK(c, hipMemset(w.pb, 0, H * 4));
       need(p, {"mix.k", "mix.v"});
@@ -1728,6 +1769,10 @@ int stack_finalize(tgx_ctx* c) {
       if ((rc = dev_alloc(c, &run.pool, ke)) || (rc = dev_alloc(c, &run.poolV, ve))) return rc;
       HIP_OK(c, hipMemset(run.pool, 0, ke));
       HIP_OK(c, hipMemset(run.poolV, 0, ve));
+      if (layer_mix_mfma(c, l)) {
+        if ((rc = dev_alloc(c, &run.poolT, ve))) return rc;
+        HIP_OK(c, hipMemset(run.poolT, 0, ve));
+      }
     } else {
       const size_t pe = rows * (size_t)(l.kv_rank + l.rot_dim) * c->esz;
       if ((rc = dev_alloc(c, &run.pool, pe))) return rc;
@@ -1861,7 +1906,7 @@ void stack_destroy(tgx_ctx* c) {
   for (auto& r : sm->rot) fr(r.cs);
   for (auto& r : sm->runs) { fr(r.pool); fr(r.poolV); fr(r.poolT); }
   for (auto& w : sm->L) { fr(w.ln); fr(w.talk); fr(w.pb); }
-  fr(sm->w_loop); fr(sm->xcat);
+  fr(sm->w_loop); fr(sm->xcat); fr(sm->qplanes);
   fr(sm->mixed); fr(sm->lora); fr(sm->rec_in);
   fr(sm->head); fr(sm->norm_g); fr(sm->a2); fr(sm->ytmp); fr(sm->ysh); fr(sm->sgw); fr(sm->vfirst); fr(sm->hs);
   fr(sm->final_norm); fr(sm->freq); fr(sm->tbl_dev); fr(sm->meta_dev); fr(sm->x); fr(sm->xs); fr(sm->a); fr(sm->proj); fr(sm->ql); fr(sm->lat); fr(sm->o); fr(sm->selw);
