@@ -7,7 +7,7 @@
 //   affine_seam_kernel         x += mult * LN_b(sublayer output) and the next sublayer's LN_a input, the experts' combine folded in
 //   sigmoid_mix_attn_kernel    a token against the window of its keys in the pool: sigmoid(score + bias) per head, weights mixed across heads, value sums
 //   sigmoid_mix_merge_kernel   adds up the partial sums of a window divided between workgroups, applies the output gate
-//   sigmoid_mix_mfma_kernel    the same attention for portions of prompts on the matrix cores
+//   (kernels/stack_mix_mfma.h holds the same attention for portions of prompts on the matrix cores)
 #pragma once
 #include "stack.h"
 
@@ -145,7 +145,8 @@ __global__ __launch_bounds__(256) void sigmoid_mix_attn_kernel(StepMeta m, MixAt
       const float* qg = s_q + (size_t)g * a.dim;
       float s = 0.f;
       if (VEC) {
-        for (int d = 0; d < a.dim; d += 8) {
+#pragma unroll 4
+        for (int d = 0; d < a.dim; d += 8) {      // (several slices in flight: a step of few tokens is bound by the latency of these loads)
           float f[8];
           slice_unpack<DT>(load_slice<DT>(kc, (size_t)(d >> 3)), f);
           const f32x4 qa = *reinterpret_cast<const f32x4*>(qg + d), qb = *reinterpret_cast<const f32x4*>(qg + d + 4);
@@ -171,6 +172,7 @@ __global__ __launch_bounds__(256) void sigmoid_mix_attn_kernel(StepMeta m, MixAt
       __syncthreads();
     }
     const float* sw = a.talk ? s_w2 : s_w;
+#pragma unroll 4
     for (int jj = 0; jj < nk; jj++) {
       const elem_t<DT>* vr = pv + (size_t)s_slot[jj] * vd;
 #pragma unroll
@@ -191,145 +193,10 @@ __global__ __launch_bounds__(256) void sigmoid_mix_merge_kernel(MixAttnArgs a) {
   const int O = a.heads * a.vdim;
   for (int o = threadIdx.x + 256 * blockIdx.y; o < O; o += 256 * gridDim.y) {
     float v = 0.f;
+#pragma unroll 8
     for (int s = 0; s < a.nsplit; s++) v += a.part[(t * a.nsplit + s) * O + o];
     a.out[t * a.ldo + o] = a.gate ? v / (1.0f + expf(-a.gate[t * a.ldg + o])) : v;
   }
-}
-
-// ---- the same attention on the matrix cores (16-bit storage; dim a multiple of 16, vdim a multiple of 32 up to 128, 1 / 2 / 4 / 8 query heads per key /
-// value head).  A workgroup owns 32 consecutive tokens of one entry and ONE key / value head c, and walks the keys its tokens see in tiles of 32:
-//   1. S_g = Q_g K_kv(g)^T for EVERY query head g (the mix needs them all), the heads dealt to the four waves; mask and sigmoid in registers, the
-//      weights to LDS in fp32.  The queries come as two 16-bit terms (one with option act.round16) from planes the append kernel writes.
-//   2. the mixed weights of the group's own heads, w'_h = sum_g talk[h][g] w_g: every thread takes four keys of one token, reads the tile of every head
-//      once and keeps the group's sums; they go back to LDS as two 16-bit terms
-//   3. O_h += w'_h V_c: every wave owns 32 value columns; its B operand comes from the transposed copy of the value page, shared by the group's heads
-// Step 1 is done once per key / value head (the workgroups of a token tile do not exchange anything): kv_heads times the score arithmetic, in exchange
-// for accumulators that fit the register file.  Key tiles never straddle a page (pages hold a multiple of 32 tokens).
-struct MixMfmaArgs {
-  const bf16_t* qh; const bf16_t* ql;   // [T][heads * dim]: the unit queries as 16-bit terms
-  const void* poolK;                    // [pages][page][kv_heads * dim]
-  const void* poolVT;                   // [pages][kv_heads * vdim][page]
-  const float* pb; const float* talk;   // as MixAttnArgs
-  const float* gate; long long ldg;
-  float* out; long long ldo;
-  int heads, kv_heads, dim, vdim, terms;
-  float scale;
-  int mask_kind, mask_size;
-};
-constexpr int MIXM_LDW = 36;            // floats per row of a weight tile in LDS (16-byte aligned rows)
-inline size_t mix_mfma_lds_bytes(int heads, int qpg) { return (size_t)heads * 32 * MIXM_LDW * 4 + (size_t)qpg * 2 * 32 * 40 * 2 + (size_t)qpg * heads * 4 + (size_t)heads * 4; }
-template <int DT, int QPG>
-__global__ __launch_bounds__(256) void sigmoid_mix_mfma_kernel(StepMeta m, MixMfmaArgs a) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];
-  const int H = a.heads;
-  float* s_w = reinterpret_cast<float*>(s_raw);                                  // [H][32][MIXM_LDW]
-  bf16_t* s_ph = reinterpret_cast<bf16_t*>(s_w + (size_t)H * 32 * MIXM_LDW);    // [QPG][32][40]
-  bf16_t* s_pl = s_ph + QPG * 32 * 40;
-  float* s_t = reinterpret_cast<float*>(s_pl + QPG * 32 * 40);                   // [QPG][H]: the rows of the mixing matrix for this group's heads
-  float* s_pb = s_t + QPG * H;                                                   // [H]
-  const int e = blockIdx.y, c = blockIdx.z;
-  const int cnt = m.ent_count[e], start = m.ent_start[e], slot = m.ent_row[e];
-  const int t0 = blockIdx.x * 32;
-  if (t0 >= cnt) return;
-  const int past = m.tok_pos[start];
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, half = lane >> 5, l31 = lane & 31;
-  const int kmax = past + min(t0 + 31, cnt - 1) + 1;
-  const int k0 = first_key(past + t0, a.mask_kind, a.mask_size) & ~31;
-  const int page = 1 << m.page_shift, kd = a.kv_heads * a.dim, vd = a.kv_heads * a.vdim, qd = H * a.dim;
-  const bf16_t* poolK = reinterpret_cast<const bf16_t*>(a.poolK);
-  const bf16_t* poolVT = reinterpret_cast<const bf16_t*>(a.poolVT);
-  for (int i = tid; i < QPG * H; i += 256) { const int hq = i / H, g = i - hq * H; s_t[i] = a.talk ? a.talk[(size_t)(c * QPG + hq) * H + g] : (g == c * QPG + hq ? 1.f : 0.f); }
-  for (int i = tid; i < H; i += 256) s_pb[i] = a.pb ? a.pb[i] : 0.f;
-  // this lane's token as the A operand's row of step 1
-  const size_t qrow = ((size_t)start + (size_t)min(t0 + l31, cnt - 1)) * qd + 8 * half;
-  // step 2's share: token srow, keys kq .. kq + 3 of the tile
-  const int srow = tid >> 3, kq = 4 * (tid & 7);
-  const bool wave_cols = 32 * wv < a.vdim;      // this wave has value columns
-  f32x16 acc[QPG];
-#pragma unroll
-  for (int hq = 0; hq < QPG; hq++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) acc[hq][r] = 0.f;
-  const int ksteps = a.dim >> 4;
-  for (int kt = k0; kt < kmax; kt += 32) {
-    const size_t pg = (size_t)m.tbl[(size_t)slot * m.tbl_stride + (kt >> m.page_shift)];
-    const int off = kt & (page - 1);
-    // 1. scores, mask and sigmoid of this wave's heads
-    for (int g = wv; g < H; g += 4) {
-      const bf16_t* kp = poolK + ((pg << m.page_shift) + off + l31) * (size_t)kd + (size_t)(g / QPG) * a.dim + 8 * half;
-      const bf16_t* qhp = a.qh + qrow + (size_t)g * a.dim;
-      const bf16_t* qlp = a.ql + qrow + (size_t)g * a.dim;
-      f32x16 s;
-#pragma unroll
-      for (int r = 0; r < 16; r++) s[r] = 0.f;
-      for (int kk = 0; kk < ksteps; kk++) {
-        const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(kp + 16 * kk));
-        s = mfma16<DT>(__builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(qhp + 16 * kk)), b, s);
-        if (a.terms > 1) s = mfma16<DT>(__builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(qlp + 16 * kk)), b, s);
-      }
-      const float bias = s_pb[g];
-      const int key = kt + l31;
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int ri = (r & 3) + 8 * (r >> 2) + 4 * half, p = past + t0 + ri;
-        const bool see = t0 + ri < cnt && key <= p && key >= first_key(p, a.mask_kind, a.mask_size);
-        s_w[((size_t)g * 32 + ri) * MIXM_LDW + l31] = see ? 1.0f / (1.0f + expf(-fmaf(s[r], a.scale, bias))) : 0.f;
-      }
-    }
-    __syncthreads();
-    // 2. the group's mixed weights
-    {
-      float mx[QPG][4];
-#pragma unroll
-      for (int hq = 0; hq < QPG; hq++)
-#pragma unroll
-        for (int k = 0; k < 4; k++) mx[hq][k] = 0.f;
-      for (int g = 0; g < H; g++) {
-        const f32x4 w4 = *reinterpret_cast<const f32x4*>(&s_w[((size_t)g * 32 + srow) * MIXM_LDW + kq]);
-#pragma unroll
-        for (int hq = 0; hq < QPG; hq++) {
-          const float tw = s_t[hq * H + g];
-#pragma unroll
-          for (int k = 0; k < 4; k++) mx[hq][k] = fmaf(tw, w4[k], mx[hq][k]);
-        }
-      }
-#pragma unroll
-      for (int hq = 0; hq < QPG; hq++) {
-        bf16_t ph[4], pl[4];
-#pragma unroll
-        for (int k = 0; k < 4; k++) split16<DT>(mx[hq][k], ph[k], pl[k]);
-        *reinterpret_cast<u32x2*>(&s_ph[(hq * 32 + srow) * 40 + kq]) = u32x2{(unsigned int)ph[0] | ((unsigned int)ph[1] << 16), (unsigned int)ph[2] | ((unsigned int)ph[3] << 16)};
-        *reinterpret_cast<u32x2*>(&s_pl[(hq * 32 + srow) * 40 + kq]) = u32x2{(unsigned int)pl[0] | ((unsigned int)pl[1] << 16), (unsigned int)pl[2] | ((unsigned int)pl[3] << 16)};
-      }
-    }
-    __syncthreads();
-    // 3. O_h += w'_h V_c on this wave's 32 value columns
-    if (wave_cols) {
-      const bf16_t* tp = poolVT + ((pg * vd + (size_t)(c * a.vdim + 32 * wv + l31)) << m.page_shift) + off + 8 * half;
-      const bf16x8 b0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(tp)), b1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(tp + 16));
-#pragma unroll
-      for (int hq = 0; hq < QPG; hq++) {
-        const bf16_t* pa = &s_ph[(hq * 32 + l31) * 40 + 8 * half];
-        const bf16_t* pl = &s_pl[(hq * 32 + l31) * 40 + 8 * half];
-        acc[hq] = mfma16<DT>(*reinterpret_cast<const bf16x8*>(pa), b0, acc[hq]);
-        acc[hq] = mfma16<DT>(*reinterpret_cast<const bf16x8*>(pa + 16), b1, acc[hq]);
-        if (a.terms > 1) {
-          acc[hq] = mfma16<DT>(*reinterpret_cast<const bf16x8*>(pl), b0, acc[hq]);
-          acc[hq] = mfma16<DT>(*reinterpret_cast<const bf16x8*>(pl + 16), b1, acc[hq]);
-        }
-      }
-    }
-  }
-  if (!wave_cols) return;
-#pragma unroll
-  for (int hq = 0; hq < QPG; hq++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int ri = (r & 3) + 8 * (r >> 2) + 4 * half;
-      if (t0 + ri >= cnt) continue;
-      const size_t tk = (size_t)start + t0 + ri, o = (size_t)(c * QPG + hq) * a.vdim + 32 * wv + l31;
-      a.out[tk * a.ldo + o] = a.gate ? acc[hq][r] / (1.0f + expf(-a.gate[tk * a.ldg + o])) : acc[hq][r];
-    }
 }
 
 }  // namespace tgx

@@ -113,9 +113,10 @@ struct StackModel {
 };
 
 // stack_gqa.hip
-namespace tgx { struct StepMeta; struct GqaMfmaArgs; }
+namespace tgx { struct StepMeta; struct GqaMfmaArgs; struct MixMfmaArgs; }
 bool gqa_mfma_shapes_ok(int dt, int dim, int vdim, int page_shift, long long ldq);
 void launch_gqa_mfma(tgx_ctx* c, const tgx::StepMeta& m, const tgx::GqaMfmaArgs& a, dim3 grid, bool split);
+void launch_mix_mfma(tgx_ctx* c, const tgx::StepMeta& m, const tgx::MixMfmaArgs& a, dim3 grid);      // kernels/stack_mix_mfma.h
 
 int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int device_ordinal, tgx_ctx** out_ctx);
 int stack_upload(tgx_ctx* c, const char* name, const void* host, const int64_t* shape, int nd, int src_dtype);

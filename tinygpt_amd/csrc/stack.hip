@@ -17,6 +17,7 @@
 #include "kernels/stack_gqa_mfma.h"
 #include "kernels/stack_rec.h"
 #include "kernels/stack_loop.h"
+#include "kernels/stack_mix_mfma.h"
 
 int upload_param_ext(tgx_ctx* c, ebyte* dst, const void* host, int64_t n, int src_dtype);      // abi.hip
 
@@ -724,22 +725,6 @@ bool layer_mix_mfma(const tgx_ctx* c, const tgx_layer_desc& l) {
   return c->dt != tgx::DT_F32 && l.dim % 16 == 0 && l.vdim % 32 == 0 && l.vdim <= 128 && (qpg == 1 || qpg == 2 || qpg == 4 || qpg == 8) && c->stack->page_shift >= 5 &&
          tgx::mix_mfma_lds_bytes(l.heads, qpg) <= MIX_ATTN_MAX_LDS;
 }
-template <int DT>
-void launch_mix_mfma_t(tgx_ctx* c, const tgx::StepMeta& m, const tgx::MixMfmaArgs& a, dim3 grid) {
-  const int qpg = a.heads / a.kv_heads;
-  const size_t lds = tgx::mix_mfma_lds_bytes(a.heads, qpg);
-  auto go = [&](auto Q) {
-    constexpr int QPG = decltype(Q)::value;
-    auto* fn = &tgx::sigmoid_mix_mfma_kernel<DT, QPG>;
-    if (lds > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipLaunchKernelGGL(fn, grid, dim3(256), lds, c->stream, m, a);
-  };
-  if (qpg == 1) go(std::integral_constant<int, 1>{});
-  else if (qpg == 2) go(std::integral_constant<int, 2>{});
-  else if (qpg == 4) go(std::integral_constant<int, 4>{});
-  else go(std::integral_constant<int, 8>{});
-}
-
 int run_affine_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const StackRun& run, int T, int S, int max_keys, int max_count) {
   StackModel* sm = c->stack;
   const tgx_layer_desc& ld = w.d;
@@ -761,7 +746,7 @@ int run_affine_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, con
     ma.gate = ld.gate_kind == 1 ? sm->proj + qd + kd + kvv : nullptr; ma.ldg = nin; ma.out = sm->o; ma.ldo = vd;
     ma.heads = H; ma.kv_heads = G; ma.dim = ld.dim; ma.vdim = ld.vdim; ma.terms = c->act16 ? 1 : 2; ma.scale = ld.scale; ma.mask_kind = ld.mask_kind; ma.mask_size = ld.mask_size;
     const dim3 grid((max_count + 31) / 32, S, G);
-    if (c->dt == tgx::DT_F16) launch_mix_mfma_t<tgx::DT_F16>(c, m, ma, grid); else launch_mix_mfma_t<tgx::DT_BF16>(c, m, ma, grid);
+    launch_mix_mfma(c, m, ma, grid);
     tgx::StackGemmArgs go{};
     go.A = sm->o; go.lda = vd; go.B = w.w_o; go.ldb = vd; go.C = sm->yd; go.ldc = W; go.M = T; go.N = W; go.K = vd; go.scale = 1.f;
     launch_gemm(c, go, tgx::SG_STORE, 1);
