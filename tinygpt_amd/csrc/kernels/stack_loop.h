@@ -90,7 +90,8 @@ __global__ __launch_bounds__(256) void affine_seam_kernel(AffineSeamArgs a) {
 // One workgroup per token (and per share of its keys in the split form).  Keys are taken KT at a time:
 //   scores   the tile's (key, head) pairs are dealt to the threads: a key row against the head's query (queries in LDS, read as broadcasts), sigmoid
 //   mix      the pairs again: a pair's mixed weight from its key's `heads` weights in LDS
-//   values   a thread owns NPT output channels (head, c): it walks the tile's keys, reading weights from LDS and value rows coalesced from the pool
+//   values   a thread owns NPT output channels (head, c), or NPT slices of eight channels where rows are 16-byte aligned (VEC): it walks the tile's keys,
+//            reading weights from LDS and value rows coalesced from the pool
 // Nothing is normalised, so the shares of a divided window are simply added (sigmoid_mix_merge_kernel, in split order).
 struct MixAttnArgs {
   const float* q; long long ldq;        // head h of token t at q + t * ldq + h * dim
@@ -123,12 +124,16 @@ __global__ __launch_bounds__(256) void sigmoid_mix_attn_kernel(StepMeta m, MixAt
   const int kd = G * a.dim, vd = G * a.vdim, O = H * a.vdim, pmask = (1 << m.page_shift) - 1;
   const elem_t<DT>* pk = reinterpret_cast<const elem_t<DT>*>(a.poolK);
   const elem_t<DT>* pv = reinterpret_cast<const elem_t<DT>*>(a.poolV);
-  float acc[NPT];
-  int oh[NPT], ov[NPT];      // the output channel's head and its column in a value row
+  // a thread's outputs: NPT channels (tid + 256 n), or with VEC NPT slices of eight neighbouring channels of one head (slice tid + 256 n)
+  constexpr int CW = VEC ? 8 : 1;
+  float acc[NPT][CW];
+  int oh[NPT], ov[NPT];      // the output's head and its (first) column in a value row
 #pragma unroll
   for (int n = 0; n < NPT; n++) {
-    const int o = tid + 256 * n, h = o < O ? o / a.vdim : 0;
-    acc[n] = 0.f; oh[n] = h; ov[n] = (h / qpg) * a.vdim + (o < O ? o - h * a.vdim : 0);
+    const int o = (tid + 256 * n) * CW, h = o < O ? o / a.vdim : 0;
+#pragma unroll
+    for (int e = 0; e < CW; e++) acc[n][e] = 0.f;
+    oh[n] = h; ov[n] = (h / qpg) * a.vdim + (o < O ? o - h * a.vdim : 0);
   }
   for (int kb = k0; kb < k1; kb += KT) {
     const int nk = min(KT, k1 - kb);
@@ -176,17 +181,27 @@ __global__ __launch_bounds__(256) void sigmoid_mix_attn_kernel(StepMeta m, MixAt
     for (int jj = 0; jj < nk; jj++) {
       const elem_t<DT>* vr = pv + (size_t)s_slot[jj] * vd;
 #pragma unroll
-      for (int n = 0; n < NPT; n++)
-        if (tid + 256 * n < O) acc[n] = fmaf(sw[(size_t)oh[n] * KT + jj], elem_to_f32<DT>(vr[ov[n]]), acc[n]);
+      for (int n = 0; n < NPT; n++) {
+        if ((tid + 256 * n) * CW >= O) continue;
+        const float wt = sw[(size_t)oh[n] * KT + jj];
+        if constexpr (VEC) {
+          float f[8];
+          slice_unpack<DT>(load_slice<DT>(vr + ov[n], 0), f);
+#pragma unroll
+          for (int e = 0; e < 8; e++) acc[n][e] = fmaf(wt, f[e], acc[n][e]);
+        } else acc[n][0] = fmaf(wt, elem_to_f32<DT>(vr[ov[n]]), acc[n][0]);
+      }
     }
   }
 #pragma unroll
-  for (int n = 0; n < NPT; n++) {
-    const int o = tid + 256 * n;
-    if (o >= O) continue;
-    if (SPLIT) a.part[((size_t)t * a.nsplit + blockIdx.y) * O + o] = acc[n];
-    else a.out[(size_t)t * a.ldo + o] = a.gate ? acc[n] / (1.0f + expf(-a.gate[(size_t)t * a.ldg + o])) : acc[n];
-  }
+  for (int n = 0; n < NPT; n++)
+#pragma unroll
+    for (int e = 0; e < CW; e++) {
+      const int o = (tid + 256 * n) * CW + e;
+      if (o >= O) continue;
+      if (SPLIT) a.part[((size_t)t * a.nsplit + blockIdx.y) * O + o] = acc[n][e];
+      else a.out[(size_t)t * a.ldo + o] = a.gate ? acc[n][e] / (1.0f + expf(-a.gate[(size_t)t * a.ldg + o])) : acc[n][e];
+    }
 }
 __global__ __launch_bounds__(256) void sigmoid_mix_merge_kernel(MixAttnArgs a) {
   const size_t t = blockIdx.x;

@@ -696,20 +696,25 @@ int run_layers_joint(tgx_ctx* c, const MetaPtrs& mp, int T, int S, int max_keys,
 // kernel applies the norm behind a sublayer, the residual add and the norm in front of the next one.
 template <int DT, bool SPLIT>
 void launch_mix_attn_t(tgx_ctx* c, const tgx::StepMeta& m, const tgx::MixAttnArgs& a, dim3 grid, size_t lds, bool vec) {
-  const int npt = (a.heads * a.vdim + 255) / 256;
+  const int npt = (a.heads * a.vdim / (vec ? 8 : 1) + 255) / 256;      // outputs per thread: channels, or slices of eight
   auto go = [&](auto N, auto V) {
     constexpr int NPT = decltype(N)::value; constexpr bool VEC = decltype(V)::value;
     auto* fn = &tgx::sigmoid_mix_attn_kernel<DT, NPT, VEC, SPLIT>;
     if (lds > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(fn, grid, dim3(256), lds, c->stream, m, a);
   };
-  auto gv = [&](auto N) { if (vec) go(N, std::true_type{}); else go(N, std::false_type{}); };
-  if (npt <= 1) gv(std::integral_constant<int, 1>{});
-  else if (npt <= 2) gv(std::integral_constant<int, 2>{});
-  else if (npt <= 4) gv(std::integral_constant<int, 4>{});
-  else if (npt <= 8) gv(std::integral_constant<int, 8>{});
-  else if (npt <= 16) gv(std::integral_constant<int, 16>{});
-  else gv(std::integral_constant<int, 32>{});
+  if (vec) {      // slices of eight channels: at most MIX_ATTN_MAX_OUT / 8 / 256 = 4 per thread
+    if (npt <= 1) go(std::integral_constant<int, 1>{}, std::true_type{});
+    else if (npt <= 2) go(std::integral_constant<int, 2>{}, std::true_type{});
+    else go(std::integral_constant<int, 4>{}, std::true_type{});
+    return;
+  }
+  if (npt <= 1) go(std::integral_constant<int, 1>{}, std::false_type{});
+  else if (npt <= 2) go(std::integral_constant<int, 2>{}, std::false_type{});
+  else if (npt <= 4) go(std::integral_constant<int, 4>{}, std::false_type{});
+  else if (npt <= 8) go(std::integral_constant<int, 8>{}, std::false_type{});
+  else if (npt <= 16) go(std::integral_constant<int, 16>{}, std::false_type{});
+  else go(std::integral_constant<int, 32>{}, std::false_type{});
 }
 constexpr int MIX_ATTN_MAX_OUT = 32 * 256;            // heads * vdim of the sigmoid attention (output channels per thread <= 32)
 constexpr size_t MIX_ATTN_MAX_LDS = 144 * 1024;
@@ -758,7 +763,7 @@ int run_affine_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, con
   aa.heads = H; aa.kv_heads = G; aa.dim = ld.dim; aa.vdim = ld.vdim; aa.scale = ld.scale; aa.mask_kind = ld.mask_kind; aa.mask_size = ld.mask_size;
   aa.kt = mix_attn_tile_keys(H, ld.dim);
   const size_t lds = tgx::mix_attn_lds_bytes(H, ld.dim, aa.kt);
-  const bool vec = ld.dim % 8 == 0;
+  const bool vec = ld.dim % 8 == 0 && ld.vdim % 8 == 0;
   const int span = ld.mask_kind == tgx::MASK_CAUSAL ? max_keys : std::min(max_keys, ld.mask_size);
   int nsplit = 1;
   if (span >= std::min(sm->gqa_split_min_keys, 128) && (long long)T < c->num_cus) {      // few tokens and a long span: the keys are divided between workgroups
