@@ -117,10 +117,11 @@ MECH = {
     "loop_from_the_first_layer": ([lat(dense()), attn(moe())], (0, 1, 3)),
     "loop_over_everything": ([attn(dense()), lat()], (0, 2, 4)),
     "loop_to_the_last_layer": ([attn(), lat(dense()), attn(moe())], (1, 3, 2)),
+    "wide_stream": ([attn(dense(8)), lat()], (1, 2, 2)),                               # a width beyond what the seam keeps in registers
     "ragged_sizes": ([attn(dense(19), heads=6, kv_heads=3, dim=5, vdim=7), lat(moe(experts=9, top=4, groups=(3, 2), ff=11, shared=3), heads=5, dim=7, rot_dim=6, vdim=3, kv_rank=13)], (0, 2, 2)),
     "deep": ([attn(dense()), lat(moe()), attn(moe(groups=None, shared=0)), lat(dense(9)), attn(), lat(), attn(dense())], (2, 6, 3)),
 }
-EXTRA = {"ragged_sizes": dict(width=27, vocab=53), "wide_heads": dict(width=40), "deep": dict(mult=1.0, scale=1.0), "many_heads": dict(width=40)}
+EXTRA = {"ragged_sizes": dict(width=27, vocab=53), "wide_heads": dict(width=40), "deep": dict(mult=1.0, scale=1.0), "many_heads": dict(width=40), "wide_stream": dict(width=4104)}
 SEEDS = {"deep": 5}      # (with the default seed two router scores of one token lie closer than bf16 rounding: the choice, a discrete one, flips)
 
 

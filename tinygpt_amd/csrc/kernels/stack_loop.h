@@ -63,11 +63,47 @@ struct AffineSeamArgs {
   float* out;                // [T][W]
   int W; float eps;
 };
+constexpr int SEAM_REG = 16;      // widths up to 256 * SEAM_REG keep a token's row in registers between the passes (same sums in the same order as the scratch form)
 __global__ __launch_bounds__(256) void affine_seam_kernel(AffineSeamArgs a) {
   __shared__ float s4[4];
   const size_t t = blockIdx.x;
-  float* yt = a.ytmp + t * a.W;
   float* xt = a.x + t * a.W;
+  if (a.W <= 256 * SEAM_REG) {
+    float v[SEAM_REG], s = 0.f;
+#pragma unroll
+    for (int k = 0; k < SEAM_REG; k++) {
+      const int c = threadIdx.x + 256 * k;
+      float y = 0.f;
+      if (c < a.W) {
+        for (int j = 0; j < a.top; j++) y += a.y[(t * a.top + j) * a.W + c];
+        if (a.ysh) y += a.ysh[t * a.W + c];
+        s += y;
+      }
+      v[k] = y;
+    }
+    float mean = block_sum_256(s, s4) / (float)a.W, q = 0.f;
+#pragma unroll
+    for (int k = 0; k < SEAM_REG; k++) if (threadIdx.x + 256 * k < a.W) { const float d = v[k] - mean; q = fmaf(d, d, q); }
+    float rstd = 1.0f / sqrtf(block_sum_256(q, s4) / (float)a.W + a.eps);
+    s = 0.f;
+#pragma unroll
+    for (int k = 0; k < SEAM_REG; k++) {
+      const int c = threadIdx.x + 256 * k;
+      if (c < a.W) { v[k] = fmaf(a.mult, fmaf((v[k] - mean) * rstd, a.w_post[c], a.b_post[c]), xt[c]); xt[c] = v[k]; s += v[k]; }
+    }
+    if (!a.w_next) return;
+    mean = block_sum_256(s, s4) / (float)a.W; q = 0.f;
+#pragma unroll
+    for (int k = 0; k < SEAM_REG; k++) if (threadIdx.x + 256 * k < a.W) { const float d = v[k] - mean; q = fmaf(d, d, q); }
+    rstd = 1.0f / sqrtf(block_sum_256(q, s4) / (float)a.W + a.eps);
+#pragma unroll
+    for (int k = 0; k < SEAM_REG; k++) {
+      const int c = threadIdx.x + 256 * k;
+      if (c < a.W) a.out[t * a.W + c] = fmaf((v[k] - mean) * rstd, a.w_next[c], a.b_next[c]);
+    }
+    return;
+  }
+  float* yt = a.ytmp + t * a.W;
   for (int c = threadIdx.x; c < a.W; c += 256) {
     float v = 0.f;
     for (int k = 0; k < a.top; k++) v += a.y[(t * a.top + k) * a.W + c];
