@@ -168,8 +168,9 @@ struct LatentAppendArgs {
   float* ql;
 };
 template <int DT>
-__global__ __launch_bounds__(64) void latent_append_kernel(StepMeta m, LatentAppendArgs a) {
-  const int t = blockIdx.x, lane = threadIdx.x, pos = m.tok_pos[t];
+__global__ __launch_bounds__(256) void latent_append_kernel(StepMeta m, LatentAppendArgs a) {
+  // one wave, or several (each sums the squares for itself, the stores are dealt to all threads)
+  const int t = blockIdx.x, lane = threadIdx.x & 63, pos = m.tok_pos[t], nth = blockDim.x;
   const float* s = a.src + (size_t)t * a.lds + a.col0;
   float ss = 0.f;
   for (int c = lane; c < a.rank; c += 64) ss = fmaf(s[c], s[c], ss);
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(64) void latent_append_kernel(StepMeta m, LatentApp
   const int row_w = a.rank + a.rot_dim;
   elem_t<DT>* dst = reinterpret_cast<elem_t<DT>*>(a.pool) + (((size_t)page << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1))) * row_w;
   elem_t<DT>* dstT = a.poolT ? reinterpret_cast<elem_t<DT>*>(a.poolT) + (((size_t)page * row_w) << m.page_shift) + (size_t)(pos & ((1 << m.page_shift) - 1)) : nullptr;
-  for (int c = lane; c < a.rank; c += 64) {
+  for (int c = threadIdx.x; c < a.rank; c += nth) {
     const elem_t<DT> v = f32_to_elem<DT>(s[c] * rinv * a.nw[c]);
     dst[c] = v;
     if (dstT) dstT[(size_t)c << m.page_shift] = v;
@@ -187,7 +188,7 @@ __global__ __launch_bounds__(64) void latent_append_kernel(StepMeta m, LatentApp
   if (a.rot_dim <= 0) return;
   const int half = a.rot_dims >> 1;
   // vector 0 is the shared key part, vectors 1 .. heads the queries' rotated parts; element i of a vector: a rotated pair member or a channel that passes
-  for (int i = lane; i < (a.heads + 1) * a.rot_dim; i += 64) {
+  for (int i = threadIdx.x; i < (a.heads + 1) * a.rot_dim; i += nth) {
     const int vec = i / a.rot_dim, ch = i - vec * a.rot_dim;
     const float* src = vec == 0 ? s + a.rank : a.q + (size_t)t * a.lds + (size_t)(vec - 1) * a.qstride + a.qoff;
     float v = src[ch];

@@ -802,7 +802,7 @@ int run_affine_latent(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const 
   la.src = sm->proj; la.lds = nin; la.col0 = qd; la.nw = w.lat_norm; la.pool = run.pool; la.poolT = run.poolT; la.rank = R; la.eps = sm->d.norm_eps;
   la.rot_dim = ld.rot_dim; la.rot_dims = ld.rot_dims; la.cs = w.rot >= 0 ? sm->rot[(size_t)w.rot].cs : nullptr;
   la.q = sm->proj; la.heads = H; la.qstride = qs; la.qoff = ld.dim; la.qscale = ld.scale; la.ql = sm->ql;
-  TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::latent_append_kernel<DT>, dim3(T), dim3(64), 0, c->stream, m, la))
+  TGX_DT_SWITCH(c->dt, hipLaunchKernelGGL(tgx::latent_append_kernel<DT>, dim3(T), dim3(256), 0, c->stream, m, la))
   // the plain part of every head's query into latent space: ql[t][h][0 .. R) = scale * q_plain[t][h] . ukT[h]^T
   g = tgx::StackGemmArgs{};
   g.A = sm->proj; g.lda = nin; g.a_zoff = qs; g.B = w.w_ukT; g.ldb = ld.dim; g.b_zstride = (long long)R * ld.dim; g.C = sm->ql; g.ldc = (long long)H * RR; g.c_zoff = RR;
