@@ -284,6 +284,51 @@ def test_split_keys_form_equals_the_direct_form():
     eng.close()
 
 
+# ---- other sizes: random layer lists, head counts, windows, loops and constants -------------------------------------------------------------------
+def random_config(rng):
+    layers = []
+    for _ in range(int(rng.integers(2, 6))):
+        if rng.random() < 0.6:
+            heads = int(rng.choice([2, 4, 6, 8, 12])); kv = int(rng.choice([g for g in (1, 2, 3, 4, 6) if heads % g == 0]))
+            dim = int(rng.choice([8, 16, 24, 32, 64]))
+            layer = attn(heads=heads, kv_heads=kv, dim=dim, vdim=int(rng.choice([8, 16, 32, 40])), mask={"size": int(rng.integers(1, 90))}, scale=float(rng.uniform(2.0, 12.0)) / dim ** 0.5)
+        else:
+            dim, rd = int(rng.choice([8, 16, 32])), int(rng.choice([0, 4, 8, 16]))
+            layer = lat(heads=int(rng.choice([1, 2, 3, 4, 8])), dim=dim, rot_dim=rd, vdim=int(rng.choice([8, 16, 24])), kv_rank=int(rng.choice([12, 32, 48, 112])),
+                        mask={"size": int(rng.integers(1, 90))}, scale=float((dim + rd) ** -0.5), rot={"base": float(rng.choice([100.0, 10000.0, 500000.0])), "dims": rd} if rd else None)
+        r = rng.random()
+        if r < 0.35:
+            layer["mlp"] = dense(int(rng.choice([12, 40, 100])))
+        elif r < 0.8:
+            experts = int(rng.choice([4, 6, 8, 12])); count = int(rng.choice([g for g in (1, 2, 3, 4) if experts % g == 0])); keep = int(rng.integers(1, count + 1))
+            layer["mlp"] = moe(experts=experts, top=int(rng.integers(1, min(4, keep * (experts // count)) + 1)), ff=int(rng.choice([6, 16, 24])), groups=(count, keep) if count > 1 else None,
+                               shared=int(rng.choice([0, 5, 16])))
+        layers.append(layer)
+    loop = None
+    if rng.random() < 0.8:
+        a = int(rng.integers(0, len(layers))); loop = (a, int(rng.integers(a + 1, len(layers) + 1)), int(rng.integers(1, 4)))
+    return config(layers, width=int(rng.choice([24, 40, 64, 72])), vocab=int(rng.choice([53, 131, 300])), eps=float(rng.choice([1e-5, 1e-6])), mult=float(rng.choice([0.3, 0.5, 1.0])),
+                  scale=float(rng.choice([1.0, 3.0, 8.0])), loop=loop)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_configurations(seed):
+    """whole prompts and portions of 1 .. 64 tokens against the oracle in fp32 (a router choice is discrete: with 16-bit storage a near tie may fall the other way)"""
+    rng = np.random.default_rng(1000 + seed)
+    cfg = random_config(rng)
+    eng, w = engine(cfg, "fp32", seed)
+    n = int(rng.integers(100, 200))
+    toks = tokens(cfg, n, seed)
+    want = want_of(cfg, w, toks)
+    check(run_whole(eng, "a", toks), want, "fp32", "whole")
+    got, at = [], 0
+    while at < n:
+        c = min(int(rng.choice([1, 2, 3, 17, 64])), n - at)
+        got.append(eng.step([("b", toks[at:at + c], list(range(c)))])); at += c
+    check(np.concatenate(got), want, "fp32", "portions")
+    eng.close()
+
+
 # ---- batches, slots, pages ----------------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
 def test_unequal_requests_in_one_batch(dtype):
