@@ -423,9 +423,10 @@ TGX_API int tgx_set_logits(tgx_ctx* ctx, const float* logits, int batch);
  *                  tgx_reset_row / tgx_reset_cache; max_ctx stays the per-row limit.  A call that would need a block when none is free returns TGX_ERR_CONTEXT and
  *                  changes nothing (retire a row, retry).  Results are those of the unpaged cache, bit for bit on the same kernels (tests/test_hip_paged.py);
  *                  tgx_get_option "kv.free_tokens" = the unassigned blocks' worth of tokens (-1 when unpaged)
- *   "attn.split_min", "attn.gqa_split_min", "attn.mfma", "stack.gemv", "stack.gemm_wt", "mlstm.narrow"  (layered models) keys a workgroup walks from which a step of few
+ *   "attn.split_min", "attn.gqa_split_min", "attn.mfma", "stack.gemv", "stack.gemm_wt", "mlstm.narrow", "attn.mix_groups"  (layered models) keys a workgroup walks from which a step of few
  *                  tokens divides them between workgroups (the first sets both thresholds, the second the grouped-query kernels' alone, counted in a mask's span);
- *                  0 = lane attention kernels only; 0 = few-row products on the matrix-core tiles too; forced product tile; the mLSTM scan's column split
+ *                  0 = lane attention kernels only; 0 = few-row products on the matrix-core tiles too; forced product tile; the mLSTM scan's column split;
+ *                  key / value heads per workgroup of the matrix-core sigmoid attention (1; 2 = two where their accumulators fit; 0 = two while the halved grid fills the chip)
  *   "debug.*"      experiment switches (tools/gemv_dissect.py, tools/attn_dissect.py; live only in a -DTGX_DISSECT=1 build) */
 TGX_API int tgx_set_option(tgx_ctx* ctx, const char* key, int value);
 

@@ -518,12 +518,13 @@ def test_matrix_core_attention_equals_the_lane_kernels(kind, shape, size):
     w = zo.random_tensors(cfg, shape["heads"])
     tens = {k: np.asarray(v, np.float32) for k, v in w.items()}
     mk = lambda: SlotEngine(desc=stack_desc_from_config(cfg, "bf16", max_seqs=4, max_ctx=1024, budget_tokens=2048), tensors=tens)
-    fast, slow = mk(), mk()
+    fast, slow, paired = mk(), mk(), mk()
     slow.model.set_option("attn.mfma", 0)
+    paired.model.set_option("attn.mix_groups", 2)          # two key / value heads per workgroup share one set of scores (by itself only on grids that fill the chip)
     a, b, c = tokens(cfg, 200, 1), tokens(cfg, 75, 2), tokens(cfg, 9, 3)
     want = want_of(cfg, w, a)[[0, 1, 69, 130, 131, 199]]
     outs = []
-    for eng in (fast, slow):
+    for eng in (fast, slow, paired):
         o = [eng.step([("a", a[:70], [0, 1, 69]), ("b", b[:3], [2])])]
         o.append(eng.step([("a", a[70:131], [60]), ("c", c, [8]), ("b", b[3:4], [0])]))
         o.append(eng.step([("b", b[4:], [70]), ("a", a[131:132], [0])]))
@@ -532,6 +533,7 @@ def test_matrix_core_attention_equals_the_lane_kernels(kind, shape, size):
         o.append(eng.step([("a", a[199:], [0]), ("b", [5], [0])]))
         outs.append(np.concatenate(o))
     assert np.abs(outs[0] - outs[1]).max() / np.abs(outs[1]).max() < 1e-3
+    assert np.abs(outs[0] - outs[2]).max() == 0.0                  # the same sums in the same order
     check(outs[0][[0, 1, 2, 4, 8, 9]], want, "bf16")               # a's positions 0, 1, 69, 130, 131, 199 in the order the steps returned them
     check(outs[0][[6, 7]], want_of(cfg, w, b)[[3, 74]], "bf16")
-    fast.close(); slow.close()
+    fast.close(); slow.close(); paired.close()

@@ -1247,6 +1247,7 @@ int tgx_set_option(tgx_ctx* c, const char* key, int value) {
     if (!strcmp(key, "attn.gqa_split_min")) { c->stack->gqa_split_min_keys = value; return TGX_OK; }
     if (!strcmp(key, "attn.mfma")) { c->stack->attn_mfma = value != 0; return TGX_OK; }      // 0: the lane-per-channel attention kernels for every layer
     if (!strcmp(key, "mlstm.narrow")) { c->stack->mlstm_narrow = value < 0 ? -1 : (value != 0); return TGX_OK; }      // the matrix-memory scan's column split (-1: automatic)
+    if (!strcmp(key, "attn.mix_groups")) { c->stack->mix_groups = value == 1 || value == 2 ? value : 0; return TGX_OK; }      // key / value heads per workgroup of the matrix-core sigmoid attention: 1, 2 (where they fit, whatever the grid), 0 = by the grid
     if (!strcmp(key, "stack.gemv")) { c->stack->gemv = value != 0; return TGX_OK; }      // 0: products of few rows on the matrix-core tiles too
     if (!strcmp(key, "stack.gemm_wt")) { if (value < 0 || value > 2) return set_err(c, TGX_ERR_INVALID, "stack.gemm_wt: 0, 1 or 2"); c->stack->gemm_wt = value; return TGX_OK; }
     return set_err(c, TGX_ERR_INVALID, "unknown option %s for a layered model", key);

@@ -109,6 +109,7 @@ struct StackModel {
   int attn_mfma = 1;                   // option attn.mfma: 0 keeps every layer on the lane-per-channel attention kernels
   int gemv = 1;                        // option stack.gemv: 0 sends products of few rows through the matrix-core tiles as well
   int mlstm_narrow = -1;               // option mlstm.narrow: the matrix-memory scan's columns per wave (1: eight, 0: sixteen, -1: by the step's entries and heads)
+  int mix_groups = 0;                  // option attn.mix_groups: key / value heads per workgroup of the matrix-core sigmoid attention: 1; 2 where their accumulators fit, whatever the grid; 0: 2 while the halved grid fills the chip
   int gemm_wt = 0;                     // option stack.gemm_wt: force the product's tile (1: 64 x 64, 2: 128 x 128); 0 = by the number of tiles
 };
 
@@ -117,6 +118,7 @@ namespace tgx { struct StepMeta; struct GqaMfmaArgs; struct MixMfmaArgs; }
 bool gqa_mfma_shapes_ok(int dt, int dim, int vdim, int page_shift, long long ldq);
 void launch_gqa_mfma(tgx_ctx* c, const tgx::StepMeta& m, const tgx::GqaMfmaArgs& a, dim3 grid, bool split);
 void launch_mix_mfma(tgx_ctx* c, const tgx::StepMeta& m, const tgx::MixMfmaArgs& a, dim3 grid);      // kernels/stack_mix_mfma.h
+size_t mix_mfma_wg_lds(int heads, int kv_heads);      // LDS bytes of one of its workgroups
 
 int stack_create(const tgx_stack_desc* desc, const tgx_layer_desc* layers, int device_ordinal, tgx_ctx** out_ctx);
 int stack_upload(tgx_ctx* c, const char* name, const void* host, const int64_t* shape, int nd, int src_dtype);

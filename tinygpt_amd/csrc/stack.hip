@@ -728,7 +728,7 @@ constexpr int MIX_MFMA_MIN_COUNT = 16;      // portions from this many tokens on
 bool layer_mix_mfma(const tgx_ctx* c, const tgx_layer_desc& l) {
   const int qpg = l.kv_heads > 0 ? l.heads / l.kv_heads : 0;
   return c->dt != tgx::DT_F32 && l.dim % 16 == 0 && l.vdim % 32 == 0 && l.vdim <= 128 && (qpg == 1 || qpg == 2 || qpg == 4 || qpg == 8) && c->stack->page_shift >= 5 &&
-         tgx::mix_mfma_lds_bytes(l.heads, qpg) <= MIX_ATTN_MAX_LDS;
+         mix_mfma_wg_lds(l.heads, l.kv_heads) <= MIX_ATTN_MAX_LDS;
 }
 int run_affine_attention(tgx_ctx* c, const tgx::StepMeta& m, StackLayerW& w, const StackRun& run, int T, int S, int max_keys, int max_count) {
   StackModel* sm = c->stack;

@@ -33,31 +33,50 @@ void launch_gqa_mfma(tgx_ctx* c, const tgx::StepMeta& m, const tgx::GqaMfmaArgs&
 
 // ---- sigmoid attention with mixed heads
 namespace {
-template <int DT, int QPG>
+// key / value heads per workgroup: two (half the score products) where the accumulators of their query heads, 16 registers each, still fit beside the
+// resident queries: not 8 accumulators beside 16 heads of 128 (they spill)
+bool mix_queries_resident(int heads, int dim, int acc_heads) {
+  const int hpw = (heads + 3) / 4;
+  return (dim == 64 || dim == 128) && hpw <= 4 && !(dim == 128 && hpw > 2 && acc_heads >= 8);
+}
+int mix_groups_per_wg(int heads, int kv_heads, int dim, int forced) {
+  const int qpg = heads / kv_heads;
+  if (kv_heads < 2 || qpg > 4) return 1;
+  if (forced == 1) return 1;
+  const bool res1 = mix_queries_resident(heads, dim, qpg), res2 = mix_queries_resident(heads, dim, 2 * qpg);
+  return res1 && !res2 ? 1 : 2;      // resident queries are worth more than shared scores
+}
+template <int DT, int QPG, int NG>
 void launch_mix_q(tgx_ctx* c, const tgx::StepMeta& m, const tgx::MixMfmaArgs& a, dim3 grid) {
-  const size_t lds = tgx::mix_mfma_lds_bytes(a.heads, QPG);
+  const size_t lds = tgx::mix_mfma_lds_bytes(a.heads, QPG * NG);
   auto go = [&](auto K, auto P) {
     constexpr int KS = decltype(K)::value, HPW = decltype(P)::value;
-    auto* fn = &tgx::sigmoid_mix_mfma_kernel<DT, QPG, KS, HPW>;
+    auto* fn = &tgx::sigmoid_mix_mfma_kernel<DT, QPG, KS, HPW, NG>;
     if (lds > 64 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(fn, grid, dim3(256), lds, c->stream, m, a);
   };
-  // a wave's heads stay in its registers where they fit: key sizes 64 / 128, at most 16 heads (8 at key size 128 ... 32 steps in all)
+  // a wave's heads stay in its registers where they fit: key sizes 64 / 128, at most 16 heads
   const int hpw = (a.heads + 3) / 4;
+  const bool res = mix_queries_resident(a.heads, a.dim, QPG * NG);
   using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>; using I2 = std::integral_constant<int, 2>; using I4 = std::integral_constant<int, 4>; using I8 = std::integral_constant<int, 8>;
-  if (a.dim == 128 && hpw <= 2) go(I8{}, I2{});
-  else if (a.dim == 128 && hpw <= 4) go(I8{}, I4{});
-  else if (a.dim == 64 && hpw <= 2) go(I4{}, I2{});
-  else if (a.dim == 64 && hpw <= 4) go(I4{}, I4{});
+  if (res && a.dim == 128 && hpw <= 2) go(I8{}, I2{});
+  else if (res && a.dim == 128) go(I8{}, I4{});
+  else if (res && a.dim == 64 && hpw <= 2) go(I4{}, I2{});
+  else if (res && a.dim == 64) go(I4{}, I4{});
   else go(I0{}, I1{});
 }
 }  // namespace
 
+size_t mix_mfma_wg_lds(int heads, int kv_heads) { return tgx::mix_mfma_lds_bytes(heads, heads / kv_heads * (kv_heads >= 2 && heads / kv_heads <= 4 ? 2 : 1)); }      // (the larger of its forms)
+
 void launch_mix_mfma(tgx_ctx* c, const tgx::StepMeta& m, const tgx::MixMfmaArgs& a, dim3 grid) {
   const int qpg = a.heads / a.kv_heads;
+  int ng = mix_groups_per_wg(a.heads, a.kv_heads, a.dim, c->stack->mix_groups);
+  if (ng == 2 && c->stack->mix_groups != 2 && (long long)grid.x * grid.y * ((a.kv_heads + 1) / 2) < c->num_cus) ng = 1;      // sharing the scores halves the workgroups: only while they still fill the chip
+  grid.z = (a.kv_heads + ng - 1) / ng;
   TGX_DT16_SWITCH(c->dt,
-    if (qpg == 1) launch_mix_q<DT, 1>(c, m, a, grid);
-    else if (qpg == 2) launch_mix_q<DT, 2>(c, m, a, grid);
-    else if (qpg == 4) launch_mix_q<DT, 4>(c, m, a, grid);
-    else launch_mix_q<DT, 8>(c, m, a, grid);)
+    if (qpg == 1) { if (ng == 2) launch_mix_q<DT, 1, 2>(c, m, a, grid); else launch_mix_q<DT, 1, 1>(c, m, a, grid); }
+    else if (qpg == 2) { if (ng == 2) launch_mix_q<DT, 2, 2>(c, m, a, grid); else launch_mix_q<DT, 2, 1>(c, m, a, grid); }
+    else if (qpg == 4) { if (ng == 2) launch_mix_q<DT, 4, 2>(c, m, a, grid); else launch_mix_q<DT, 4, 1>(c, m, a, grid); }
+    else launch_mix_q<DT, 8, 1>(c, m, a, grid);)
 }
